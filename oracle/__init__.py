@@ -1,0 +1,32 @@
+"""CPU oracle for the MoEspresso attention hot path.
+
+TEST INFRASTRUCTURE ONLY. Nothing in the product package imports this. Only
+the test suite, the smoke check and the CPU-baseline leg of the benchmark may
+call it, and there only as the checker.
+
+Every function restates, in NumPy, an algorithm of the reference and cites the
+reference file:line it follows. The reference cannot run outside Apple Metal
+(MLX), so the restatement is pinned by the reference's own known-answer tests,
+by closed forms and by brute force on tiny inputs (see tests/test_oracle_*.py).
+
+Parity status per function group ("pinned" = a check that a plausible mistake
+would fail; "unpinned" = only self-consistency is available):
+
+  hadamard128 / indexer_qat          pinned  (H.H=128 I vs scipy, ones KAT, lattice invariants)
+  pow2 group scale bit patterns      parity unpinned at stress exponents: the
+                                     reference keeps Metal's precise::log/exp
+                                     bits; this oracle uses correctly rounded
+                                     float32 log/exp (exactly 2^k for |k| <= 12,
+                                     a few ulp off 2^k beyond, as in the reference)
+  e4m3fn table / fp8_kv_roundtrip    pinned  (torch.float8_e4m3fn cast away from ties, table closed form)
+  indexer scores                     pinned  (64*scale KAT, 144/sqrt(128) KAT, float64 closed form)
+  score_tail reduction order         parity unpinned (MLX col_reduce/simd_sum tree is
+                                     not observable; own fixed order, value pinned by float64)
+  radix_select_topk                  pinned  (lexsort brute force, all-tie -> arange, reference KAT)
+  rope / yarn                        pinned  (reference pinned inv-freq and angle values)
+  sink attention / visit rules       pinned  (single-key+sink KAT, torch.softmax when sink=-inf,
+                                     visibility KATs, brute-force row lists)
+  q8 quantisers (affine g64)         parity unpinned (MLX mx.quantize edge rules not in the
+                                     reference tree; own documented rule, round trip bounded)
+  gqa decode / causal flash prefill  pinned  (float64 torch.softmax closed form)
+"""

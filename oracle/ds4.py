@@ -1,0 +1,750 @@
+"""NumPy restatement of the DeepSeek-V4 side of the attention hot path.
+
+TEST INFRASTRUCTURE ONLY (see oracle/__init__.py). Citations are paths under
+the reference tree, ``src/moespresso/runtime/deepseek_v4/`` unless a longer
+path is given.
+
+Two numeric modes appear below:
+
+* "f32-faithful" functions reproduce the reference's float32 operation
+  sequence (rounding after every composed op) and are compared bit-for-bit
+  with the HIP kernels that claim bit identity (QAT rows, FP8 rows, prepared
+  KV row, score tail, top-k indices).
+* "f64 truth" functions evaluate the closed form in float64 and are compared
+  within the tolerance the reference's own tests use.
+
+Transcendentals in the power-of-two group scale use correctly rounded float32
+``log``/``exp`` (evaluated in float64, rounded once to float32). The reference
+keeps whatever bits Metal's ``precise::log/exp`` give; the two agree for
+ordinary exponents and may differ by an ulp of the scale at stress exponents
+(parity unpinned there; see oracle/__init__.py).
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Mapping, Sequence
+
+import numpy as np
+
+F32 = np.float32
+
+# indexer_score_kernel.py:74-76 and model.py:725,735
+HADAMARD_SCALE = F32(0.08838834764831845)
+AMAX_FLOOR = F32(7.052966104933725e-38)
+LN2F = F32(math.log(2.0))
+E2M1_LATTICE = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], dtype=F32)
+FP8_AMAX_FLOOR = F32(1.0e-4)
+
+DS4_HEAD_DIM = 512
+DS4_ROPE_DIM = 64
+DS4_SWA_ROPE_BASE = 10000.0
+DS4_COMPRESS_ROPE_BASE = 160000.0
+DS4_YARN = {
+    "factor": 16.0,
+    "original_seq_len": 65536.0,
+    "beta_fast": 32.0,
+    "beta_slow": 1.0,
+}
+
+
+# --------------------------------------------------------------------------
+# float helpers
+# --------------------------------------------------------------------------
+
+def f32_log(x: np.ndarray) -> np.ndarray:
+    """Correctly rounded float32 natural log (float64 evaluation, one rounding)."""
+    with np.errstate(divide="ignore", invalid="ignore"):
+        return np.log(np.asarray(x, dtype=np.float64)).astype(F32)
+
+
+def f32_exp(x: np.ndarray) -> np.ndarray:
+    """Correctly rounded float32 exp (float64 evaluation, one rounding)."""
+    with np.errstate(over="ignore", under="ignore"):
+        return np.exp(np.asarray(x, dtype=np.float64)).astype(F32)
+
+
+def round_bf16(x: np.ndarray) -> np.ndarray:
+    """Round float32 to bfloat16 (nearest even) and return it widened to float32."""
+    a = np.ascontiguousarray(np.asarray(x, dtype=F32))
+    u = a.view(np.uint32).astype(np.uint64)
+    nan = np.isnan(a)
+    r = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    out = r.astype(np.uint32).view(F32).copy()
+    out[nan] = np.nan
+    return out
+
+
+def round_f16(x: np.ndarray) -> np.ndarray:
+    """Round to float16 and widen back to float32."""
+    with np.errstate(over="ignore"):
+        return np.asarray(x, dtype=F32).astype(np.float16).astype(F32)
+
+
+def _mx_maximum(a: np.ndarray, b) -> np.ndarray:
+    """MLX Maximum: NaN in ``a`` passes through (indexer_score_kernel.py:106-107)."""
+    a = np.asarray(a, dtype=F32)
+    return np.where(np.isnan(a), a, np.where(a > b, a, F32(b))).astype(F32)
+
+
+def _mx_clip(n: np.ndarray, lo: float, hi: float) -> np.ndarray:
+    """mx.clip = maximum then minimum with NaN passthrough (indexer_score_kernel.py:115-117)."""
+    n = np.asarray(n, dtype=F32)
+    n = np.where(np.isnan(n) | (n > F32(lo)), n, F32(lo))
+    n = np.where(np.isnan(n) | (n < F32(hi)), n, F32(hi))
+    return n.astype(F32)
+
+
+def pow2_group_scale(amax: np.ndarray, denom: float) -> np.ndarray:
+    """``exp(ceil(log(amax/denom)/ln2)*ln2)`` in float32.
+
+    model.py:736-737 (denom 6) and model.py:594-595 (denom 448); Metal form
+    indexer_score_kernel.py:108-109, decode_attention_kernel.py:156-157.
+    """
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        r = (np.asarray(amax, dtype=F32) / F32(denom)).astype(F32)
+        log2_scale = (f32_log(r) / LN2F).astype(F32)
+        e = (np.ceil(log2_scale).astype(F32) * LN2F).astype(F32)
+        return f32_exp(e)
+
+
+# --------------------------------------------------------------------------
+# a1/a2: indexer QAT (Hadamard-128 + e2m1 activation round trip)
+# --------------------------------------------------------------------------
+
+def hadamard128_unscaled(x: np.ndarray) -> np.ndarray:
+    """Walsh-Hadamard transform of 128-wide rows, radix-2, strides 1,2,...,64.
+
+    float32 butterflies ``(a, b) -> (a + b, a - b)`` in increasing-stride
+    order (indexer_score_kernel.py:83-95; model.py:720-725).
+    """
+    x = np.asarray(x)
+    if x.shape[-1] != 128:
+        raise ValueError("indexer QAT expects 128-wide rows")
+    y = x.astype(F32).reshape(-1, 128)
+    h = 1
+    while h < 128:
+        y = y.reshape(-1, 128 // (2 * h), 2, h)
+        a = y[:, :, 0, :]
+        b = y[:, :, 1, :]
+        y = np.stack(((a + b).astype(F32), (a - b).astype(F32)), axis=2)
+        h *= 2
+    return y.reshape(x.shape).astype(F32)
+
+
+def hadamard128(x: np.ndarray) -> np.ndarray:
+    """model.py:720-725: ``hadamard_transform(x.astype(f32), scale=128**-0.5)``."""
+    return (hadamard128_unscaled(x) * HADAMARD_SCALE).astype(F32)
+
+
+def indexer_fp4_act_roundtrip(y: np.ndarray) -> np.ndarray:
+    """e2m1 lattice round trip over 32-element groups (model.py:728-742).
+
+    Ties in the nearest-lattice search go to the first (lower) lattice value
+    (``mx.argmin``; indexer_score_kernel.py:119-128).
+    """
+    y = np.asarray(y, dtype=F32)
+    shape = y.shape
+    g = y.reshape(-1, shape[-1] // 32, 32)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        amax = np.max(np.abs(g), axis=-1, keepdims=True)  # np.max propagates NaN
+        amax = _mx_maximum(amax, AMAX_FLOOR)
+        scale = pow2_group_scale(amax, 6.0)
+        n = _mx_clip((g / scale).astype(F32), -6.0, 6.0)
+        absn = np.abs(n)
+        diff = np.abs(absn[..., None] - E2M1_LATTICE).astype(F32)
+        # argmin with NaN: every comparison is false, the first entry stays.
+        diff_for_argmin = np.where(np.isnan(diff), np.inf, diff)
+        nearest = np.argmin(diff_for_argmin, axis=-1)
+        dq = E2M1_LATTICE[nearest]
+        dq = np.where(n < 0, -dq, dq).astype(F32)
+        out = (dq * scale).astype(F32)
+    return out.reshape(shape)
+
+
+def indexer_qat(x: np.ndarray) -> np.ndarray:
+    """model.py:745-749: Hadamard-128 then the e2m1 round trip; float32 out."""
+    return indexer_fp4_act_roundtrip(hadamard128(x))
+
+
+# --------------------------------------------------------------------------
+# a10: E4M3FN KV round trip
+# --------------------------------------------------------------------------
+
+def e4m3fn_values() -> np.ndarray:
+    """The 127 non-negative finite E4M3FN values, ascending (model.py:531-540)."""
+    values = []
+    for code in range(127):
+        exp = (code >> 3) & 0x0F
+        mant = code & 0x07
+        if exp == 0:
+            values.append(float(mant) * 0.001953125)
+        else:
+            values.append((1.0 + float(mant) * 0.125) * float(2 ** (exp - 7)))
+    return np.asarray(values, dtype=F32)
+
+
+def fp8_nearest_first_wins(absn: np.ndarray) -> np.ndarray:
+    """Nearest E4M3FN value by a literal first-wins table scan (model.py:600-603)."""
+    table = e4m3fn_values()
+    absn = np.asarray(absn, dtype=F32)
+    flat = absn.reshape(-1)
+    out = np.empty_like(flat)
+    step = 1 << 14
+    for s in range(0, flat.size, step):
+        blk = flat[s:s + step]
+        diff = np.abs(blk[:, None] - table[None, :]).astype(F32)
+        diff = np.where(np.isnan(diff), np.inf, diff)
+        out[s:s + step] = table[np.argmin(diff, axis=-1)]
+    return out.reshape(absn.shape)
+
+
+def fp8_kv_roundtrip(x: np.ndarray, *, head_dim: int = 512, rot_dim: int = 64) -> np.ndarray:
+    """E4M3FN round trip on dims [0, head_dim-rot_dim) in 64-blocks (model.py:559-609).
+
+    Input/output float32 (the reference casts back to the input dtype; the
+    caller does that). Dims [448, 512) are copied.
+    """
+    x = np.asarray(x, dtype=F32)
+    if x.shape[-1] != head_dim:
+        raise ValueError("fp8 rows expect head_dim-wide rows")
+    n_nope = head_dim - rot_dim
+    prefix = x[..., :n_nope]
+    tail = x[..., n_nope:]
+    blocks = prefix.reshape(-1, n_nope // 64, 64)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        amax = np.max(np.abs(blocks), axis=-1, keepdims=True)
+        amax = _mx_maximum(amax, FP8_AMAX_FLOOR)
+        scale = pow2_group_scale(amax, 448.0)
+        scaled = _mx_clip((blocks / scale).astype(F32), -448.0, 448.0)
+        q = fp8_nearest_first_wins(np.abs(scaled))
+        sign = np.where(scaled < 0, F32(-1.0), np.where(scaled > 0, F32(1.0), F32(0.0))).astype(F32)
+        rounded = ((sign * q).astype(F32) * scale).astype(F32).reshape(prefix.shape)
+    return np.concatenate([rounded, tail], axis=-1).astype(F32)
+
+
+# --------------------------------------------------------------------------
+# a3: decode score row
+# --------------------------------------------------------------------------
+
+def indexer_scores_f64(q_qat: np.ndarray, pooled: np.ndarray, weights: np.ndarray,
+                       scale: float) -> np.ndarray:
+    """``scores[r] = sum_h max(q_h . p_r, 0) * scale * w_h`` in float64.
+
+    indexer_score_kernel.py:176-186; composed chain model.py:1041-1046.
+    q_qat [H,128], pooled [N,128], weights [H] -> [N].
+    """
+    q = np.asarray(q_qat, dtype=np.float64)
+    p = np.asarray(pooled, dtype=np.float64)
+    w = np.asarray(weights, dtype=np.float64).reshape(-1)
+    raw = q @ p.T
+    return (np.maximum(raw, 0.0) * float(scale) * w[:, None]).sum(axis=0)
+
+
+def fused_qat_indexer_scores(q: np.ndarray, pooled_qat: np.ndarray, weights: np.ndarray,
+                             scale: float) -> np.ndarray:
+    """a3 with the reference argument layout (indexer_score_kernel.py:354-409).
+
+    q ``[1,H,1,128]`` any float, pooled_qat f32 ``[1,N,128]``, weights f32
+    ``[1,1,H]`` -> float64 ``[N]`` (callers compare with rtol=atol=1e-5, the
+    reference's own bar, test_deepseek_v4_indexer_score_kernel.py:137-163).
+    """
+    q = np.asarray(q)
+    n_heads = q.shape[1]
+    qq = indexer_qat(q.reshape(n_heads, 128).astype(F32))
+    return indexer_scores_f64(qq, np.asarray(pooled_qat).reshape(-1, 128),
+                              np.asarray(weights).reshape(-1), scale)
+
+
+# --------------------------------------------------------------------------
+# a5: fused score tail
+# --------------------------------------------------------------------------
+
+def score_tail(scores: np.ndarray, weights_raw: np.ndarray, params: np.ndarray, *,
+               scale: float) -> np.ndarray:
+    """relu, score scale, head-weight cast+scale, head sum, pad, negate.
+
+    indexer_score_kernel.py:460-491. ``scores`` f32 ``[H, C]``; ``weights_raw``
+    ``[H]`` already widened to f32 exactly (f16/bf16 -> f32 is exact);
+    ``params[1]`` = valid column count. Every step rounds to float32. Lane
+    ``l`` (0..31) adds heads ``l, l+32`` in order starting from +0.0; the 32
+    partials are combined by an xor butterfly (offsets 16, 8, 4, 2, 1). The
+    reference's ``simd_sum`` tree is not observable, so that last order is
+    this build's own rule (parity unpinned for the reduction order only).
+    """
+    s = np.asarray(scores, dtype=F32)
+    n_heads, capacity = s.shape
+    w = np.asarray(weights_raw, dtype=F32).reshape(n_heads)
+    head_norm = F32(float(int(n_heads) ** -0.5))
+    score_scale = F32(scale)
+    valid = min(int(np.asarray(params).reshape(-1)[1]), capacity)
+    with np.errstate(invalid="ignore", over="ignore"):
+        wn = (w * head_norm).astype(F32)
+        partial = np.zeros((32, capacity), dtype=F32)
+        for h in range(n_heads):
+            t = s[h]
+            t = np.where(np.isnan(t), t, np.where(t > 0, t, F32(0.0))).astype(F32)
+            t = (t * score_scale).astype(F32)
+            t = (t * wn[h]).astype(F32)
+            partial[h % 32] = (partial[h % 32] + t).astype(F32)
+        off = 16
+        while off >= 1:
+            partial = (partial[:off] + partial[off:2 * off]).astype(F32)
+            off //= 2
+        total = partial[0]
+    neg = np.where(np.arange(capacity) < valid, -total, F32(np.inf)).astype(F32)
+    return neg
+
+
+def decode_step_params(offset: int, pool_rows: int) -> np.ndarray:
+    """fixed_decode_state.py:186-195: int32 ``[offset, pool_rows]``."""
+    return np.asarray([int(offset), int(pool_rows)], dtype=np.int32)
+
+
+def pad_scores_to_capacity(scores: np.ndarray, pool_rows: int) -> np.ndarray:
+    """fixed_decode_state.py:198-206: columns >= pool_rows become -inf."""
+    s = np.asarray(scores, dtype=F32).copy()
+    s[..., int(pool_rows):] = -np.inf
+    return s
+
+
+# --------------------------------------------------------------------------
+# A3: deterministic top-k
+# --------------------------------------------------------------------------
+
+def score_key(s: np.ndarray) -> np.ndarray:
+    """Monotone float32 -> uint32 map (decode_attention_kernel.py:115-120)."""
+    u = np.ascontiguousarray(np.asarray(s, dtype=F32)).view(np.uint32)
+    return np.where(u & np.uint32(0x80000000), ~u, u | np.uint32(0x80000000)).astype(np.uint32)
+
+
+def radix_select_topk(scores: np.ndarray, topk: int) -> np.ndarray:
+    """Four-pass MSB radix select + ordered emission (decode_attention_kernel.py:295-375).
+
+    Returns int32 ``[topk]``: rows whose key is strictly above the threshold
+    in ascending row order, then the lowest-index rows tied with it.
+    Requires ``0 < topk <= n_rows``.
+    """
+    keys = score_key(np.asarray(scores, dtype=F32).reshape(-1))
+    n = keys.size
+    topk = int(topk)
+    if not 0 < topk <= n:
+        raise ValueError("topk must be in (0, n_rows]")
+    prefix = np.uint32(0)
+    need = topk
+    for p in range(4):
+        shift = 24 - 8 * p
+        mask_hi = np.uint32(0) if p == 0 else np.uint32((0xFFFFFFFF << (shift + 8)) & 0xFFFFFFFF)
+        live = (keys & mask_hi) == prefix
+        hist = np.bincount(((keys[live] >> np.uint32(shift)) & np.uint32(0xFF)).astype(np.int64),
+                           minlength=256)
+        b = 255
+        while True:
+            c = int(hist[b])
+            if c >= need or b == 0:
+                break
+            need -= c
+            b -= 1
+        prefix = np.uint32(prefix | np.uint32(b << shift))
+    threshold = prefix
+    need_ties = need
+    above = np.flatnonzero(keys > threshold)
+    ties = np.flatnonzero(keys == threshold)[:need_ties]
+    return np.concatenate([above, ties]).astype(np.int32)
+
+
+def topk_lexsort(scores: np.ndarray, topk: int) -> np.ndarray:
+    """Brute-force top-k: descending key, ties to the lower index.
+
+    Equals ``attention.py:305-312`` (stable argsort of ``-score``) on finite,
+    NaN-free input, and ``radix_select_topk`` as a set on any input.
+    """
+    keys = score_key(np.asarray(scores, dtype=F32).reshape(-1)).astype(np.int64)
+    order = np.lexsort((np.arange(keys.size), -keys))
+    return order[:int(topk)].astype(np.int32)
+
+
+# --------------------------------------------------------------------------
+# a18: pure closed forms of attention.py
+# --------------------------------------------------------------------------
+
+def rope_inverse_frequencies(dim: int, base: float,
+                             yarn: Mapping[str, float] | None = None) -> np.ndarray:
+    """attention.py:71-102 (float64; YaRN ramp folded into the frequencies)."""
+    if dim <= 0 or dim % 2:
+        raise ValueError("RoPE dim must be a positive even integer")
+    idx = np.arange(0, dim, 2, dtype=np.float64)
+    freqs = 1.0 / (float(base) ** (idx / dim))
+    if not yarn:
+        return freqs
+    factor = float(yarn["factor"])
+    original = float(yarn["original_seq_len"])
+    beta_fast = float(yarn.get("beta_fast", 32.0))
+    beta_slow = float(yarn.get("beta_slow", 1.0))
+    if factor <= 1.0 or original <= 0:
+        return freqs
+
+    def correction_dim(n: float) -> float:
+        return dim * math.log(original / (n * 2.0 * math.pi)) / (2.0 * math.log(base))
+
+    low = max(math.floor(correction_dim(beta_fast)), 0)
+    high = min(math.ceil(correction_dim(beta_slow)), dim - 1)
+    if low == high:
+        high += 0.001
+    ramp = (np.arange(dim // 2, dtype=np.float64) - low) / (high - low)
+    smooth = 1.0 - np.clip(ramp, 0.0, 1.0)
+    return freqs / factor * (1.0 - smooth) + freqs * smooth
+
+
+def rope_angles(positions, *, dim: int = DS4_ROPE_DIM, base: float,
+                yarn: Mapping[str, float] | None = None) -> np.ndarray:
+    """attention.py:105-114."""
+    pos = np.asarray(positions, dtype=np.float64).reshape(-1)
+    return np.outer(pos, rope_inverse_frequencies(dim, base, yarn))
+
+
+def apply_rope_tail(x: np.ndarray, positions, *, base: float,
+                    yarn: Mapping[str, float] | None = None,
+                    rope_dim: int = DS4_ROPE_DIM, inverse: bool = False) -> np.ndarray:
+    """attention.py:117-156: float64 rotation of interleaved pairs on the tail."""
+    arr = np.asarray(x)
+    out = arr.copy()
+    tail = out[..., -rope_dim:]
+    pairs = tail.astype(np.float64).reshape(*tail.shape[:-1], rope_dim // 2, 2)
+    angles = rope_angles(positions, dim=rope_dim, base=base, yarn=yarn)
+    cos, sin = np.cos(angles), np.sin(angles)
+    if inverse:
+        sin = -sin
+    bshape = (1,) * (pairs[..., 0].ndim - 2) + cos.shape
+    cos, sin = cos.reshape(bshape), sin.reshape(bshape)
+    x0, x1 = pairs[..., 0], pairs[..., 1]
+    rot = np.stack((x0 * cos - x1 * sin, x0 * sin + x1 * cos), axis=-1)
+    out[..., -rope_dim:] = rot.reshape(tail.shape).astype(out.dtype)
+    return out
+
+
+def compressed_visibility(query_positions, pool_indices, ratio: int) -> np.ndarray:
+    """attention.py:159-173: pool row k visible to q iff (k+1)*ratio <= q+1."""
+    if ratio <= 0:
+        raise ValueError("ratio must be positive")
+    q = np.asarray(query_positions, dtype=np.int64).reshape(-1)
+    k = np.asarray(pool_indices, dtype=np.int64).reshape(-1)
+    return ((k[None, :] + 1) * int(ratio)) <= (q[:, None] + 1)
+
+
+def visible_compressed_count(query_positions, ratio: int) -> np.ndarray:
+    """attention.py:176-184."""
+    if ratio <= 0:
+        raise ValueError("ratio must be positive")
+    return (np.asarray(query_positions, dtype=np.int64).reshape(-1) + 1) // int(ratio)
+
+
+def compressed_rope_positions(pool_indices, ratio: int, *, pool_base: int = 0) -> np.ndarray:
+    """attention.py:187-197."""
+    if ratio <= 0:
+        raise ValueError("ratio must be positive")
+    return int(pool_base) + np.asarray(pool_indices, dtype=np.int64).reshape(-1) * int(ratio)
+
+
+def sink_softmax_attention(scores: np.ndarray, values: np.ndarray, sinks: np.ndarray) -> np.ndarray:
+    """attention.py:200-223: softmax with a zero-value sink in the denominator."""
+    s = np.asarray(scores, dtype=np.float64)
+    v = np.asarray(values, dtype=np.float64)
+    k = np.asarray(sinks, dtype=np.float64)
+    v = np.broadcast_to(v, s.shape + (v.shape[-1],))
+    k = np.broadcast_to(k, s.shape[:-1])
+    if s.shape[-1] == 0:
+        return np.zeros(s.shape[:-1] + (v.shape[-1],), dtype=np.float64)
+    m = np.maximum(np.max(s, axis=-1), k)
+    with np.errstate(invalid="ignore"):
+        w = np.exp(s - m[..., None])
+        sw = np.exp(k - m)
+    den = np.sum(w, axis=-1) + sw
+    return np.sum(w[..., None] * v, axis=-2) / den[..., None]
+
+
+def indexer_weight_scale(index_head_dim: int = 128, n_heads: int = 64) -> float:
+    """attention.py:226-230."""
+    return (index_head_dim ** -0.5) * (n_heads ** -0.5)
+
+
+def indexer_weighted_scores(raw_scores: np.ndarray, head_weights: np.ndarray, *,
+                            index_head_dim: int = 128, n_heads: int = 64) -> np.ndarray:
+    """attention.py:233-251: relu, per-head weights, head sum, scale."""
+    raw = np.asarray(raw_scores, dtype=np.float64)
+    w = np.asarray(head_weights, dtype=np.float64)
+    return np.sum(np.maximum(raw, 0.0) * w[..., None], axis=1) * indexer_weight_scale(
+        index_head_dim, n_heads)
+
+
+def causal_indexer_topk(raw_scores, head_weights, query_positions, pool_indices, ratio: int, *,
+                        topk: int = 512, index_head_dim: int = 128, n_heads: int = 64) -> np.ndarray:
+    """attention.py:277-313: mask future blocks, stable top-k, pad with -1."""
+    pool = np.asarray(pool_indices, dtype=np.int64).reshape(-1)
+    weighted = indexer_weighted_scores(raw_scores, head_weights,
+                                       index_head_dim=index_head_dim, n_heads=n_heads)
+    scores = np.where(compressed_visibility(query_positions, pool, ratio), weighted, -np.inf)
+    width = min(int(topk), pool.shape[0])
+    out = np.full((scores.shape[0], width), -1, dtype=np.int64)
+    for i, row in enumerate(scores):
+        valid = np.flatnonzero(np.isfinite(row))
+        if valid.size == 0 or width == 0:
+            continue
+        order = valid[np.argsort(-row[valid], kind="stable")[:width]]
+        out[i, :order.size] = pool[order]
+    return out
+
+
+# --------------------------------------------------------------------------
+# A5: partial rope at element-dtype op rounding
+# --------------------------------------------------------------------------
+
+def rope_cos_sin_f32(pos: int, inv_freq: np.ndarray):
+    """theta = f32(pos) * inv_freq (float32), cos/sin correctly rounded to float32.
+
+    decode_attention_kernel.py:251-253 (``metal::precise::cos/sin``).
+    """
+    theta = (F32(pos) * np.asarray(inv_freq, dtype=F32)).astype(F32)
+    t64 = theta.astype(np.float64)
+    return np.cos(t64).astype(F32), np.sin(t64).astype(F32)
+
+
+def partial_rope_lowp(x: np.ndarray, pos: int, inv_freq: np.ndarray, *, inverse: bool = False,
+                      rnd=round_f16, rope_dim: int = DS4_ROPE_DIM) -> np.ndarray:
+    """Partial rope with every product and sum rounded to the element dtype.
+
+    decode_attention_kernel.py:136-147 and attention_seam_kernel.py:88-118.
+    ``x`` holds values already representable in the element dtype (as float32);
+    the last ``rope_dim`` channels are interleaved pairs. Returns float32
+    holding element-dtype values.
+    """
+    x = np.asarray(x, dtype=F32)
+    out = x.copy()
+    c32, s32 = rope_cos_sin_f32(pos, inv_freq)
+    c = rnd(c32)
+    s = rnd(-s32 if inverse else s32)
+    tail = x[..., -rope_dim:]
+    x0 = tail[..., 0::2]
+    x1 = tail[..., 1::2]
+    m0 = rnd((x0 * c).astype(F32))
+    m1 = rnd((x1 * s).astype(F32))
+    m2 = rnd((x0 * s).astype(F32))
+    m3 = rnd((x1 * c).astype(F32))
+    r0 = rnd((m0 - m1).astype(F32))
+    r1 = rnd((m2 + m3).astype(F32))
+    rot = np.stack((r0, r1), axis=-1).reshape(tail.shape)
+    out[..., -rope_dim:] = rot
+    return out
+
+
+# --------------------------------------------------------------------------
+# A4: indexed mixed attention (visit rules + sink softmax)
+# --------------------------------------------------------------------------
+
+def indexed_visit_rows(*, raw_cap: int, n_comp: int, topk: np.ndarray, qpos: int, last_pos: int,
+                       window: int, ratio: int, raw_start: int):
+    """Rows one query visits, in order (indexed_attention_kernel.py:120-155).
+
+    Returns ``(raw_rows, comp_rows)``: ring-buffer rows then pool rows.
+    ``last_pos`` is the absolute position of the newest raw row (``pos0`` for
+    decode). Negative ids are skipped; the first id >= visible stops the walk.
+    """
+    raw_rows = []
+    n_raw = int(raw_cap)
+    if n_raw > 0:
+        first_raw_pos = int(last_pos) + 1 - n_raw
+        raw_last_pos = first_raw_pos + n_raw - 1
+        window_first = qpos + 1 - window if (window != 0 and qpos + 1 > window) else 0
+        first = max(first_raw_pos, window_first)
+        last = min(qpos, raw_last_pos)
+        for pos in range(first, last + 1):
+            raw_rows.append((int(raw_start) + (pos - first_raw_pos)) % n_raw)
+    visible = n_comp if ratio == 0 else (qpos + 1) // ratio
+    visible = min(visible, n_comp)
+    comp_rows = []
+    for idx in np.asarray(topk).reshape(-1).tolist():
+        if idx < 0:
+            continue
+        if idx >= visible:
+            break
+        comp_rows.append(int(idx))
+    return raw_rows, comp_rows
+
+
+def attend_rows_f64(q: np.ndarray, rows: np.ndarray, sinks, scale: float,
+                    v_dim: int | None = None) -> np.ndarray:
+    """float64 sink attention of ``q [H,D]`` over ``rows [R,D]`` (V = rows[:, :v_dim])."""
+    q = np.asarray(q, dtype=np.float64)
+    rows = np.asarray(rows, dtype=np.float64)
+    v_dim = rows.shape[-1] if v_dim is None else v_dim
+    n_heads = q.shape[0]
+    if sinks is None:
+        sinks = np.full((n_heads,), -np.inf)
+    if rows.shape[0] == 0:
+        return np.zeros((n_heads, v_dim), dtype=np.float64)
+    s = (q @ rows.T) * float(scale)
+    return sink_softmax_attention(s, rows[None, :, :v_dim], np.asarray(sinks, dtype=np.float64))
+
+
+def indexed_mixed_attention_decode(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
+                                   ratio: int = 4, raw_start: int = 0) -> np.ndarray:
+    """One-token indexed mixed attention (indexed_attention_kernel.py:61-174, 1496-1568).
+
+    q f32 ``[H,512]`` (rounded to half on load, :79-82), raw_kv/comp_kv f16,
+    scale ``rsqrt(head_dim)``, sink joins max and denominator once; float64.
+    """
+    qh = round_f16(np.asarray(q, dtype=F32))
+    raw = np.asarray(raw_kv).astype(F32)
+    comp = np.asarray(comp_kv).astype(F32)
+    raw_rows, comp_rows = indexed_visit_rows(
+        raw_cap=raw.shape[0], n_comp=comp.shape[0], topk=topk, qpos=int(pos0), last_pos=int(pos0),
+        window=int(window), ratio=int(ratio), raw_start=int(raw_start))
+    rows = np.concatenate([raw[raw_rows].reshape(-1, raw.shape[1]),
+                           comp[comp_rows].reshape(-1, raw.shape[1])], axis=0)
+    return attend_rows_f64(qh, rows, sinks, float(q.shape[-1]) ** -0.5)
+
+
+def selected_rows_attention_reference(q, raw_kv, comp_kv, topk, sinks) -> np.ndarray:
+    """indexed_attention_kernel.py:2111-2130: take + concat + SDPA with f16 q and sinks."""
+    qh = round_f16(np.asarray(q, dtype=F32))
+    raw = np.asarray(raw_kv).astype(F32)
+    comp = np.asarray(comp_kv).astype(F32)
+    full = np.concatenate([raw, comp[np.asarray(topk, dtype=np.int64)]], axis=0)
+    return attend_rows_f64(qh, full, round_f16(np.asarray(sinks, dtype=F32)),
+                           float(q.shape[-1]) ** -0.5)
+
+
+def indexed_mixed_attention_prefill(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
+                                    ratio: int = 4, raw_start: int = 0) -> np.ndarray:
+    """Per-token A4 for a prefill chunk (indexed_attention_kernel.py:2030-2108, 2133-2180).
+
+    q ``[T,H,512]``, raw_kv ``[raw_cap,512]``, topk ``[T,k]`` -> float64 ``[T,H,512]``.
+    """
+    q = np.asarray(q)
+    n_tokens = q.shape[0]
+    raw = np.asarray(raw_kv).astype(F32)
+    comp = np.asarray(comp_kv).astype(F32)
+    last_pos = int(pos0) + n_tokens - 1
+    out = np.zeros(q.shape, dtype=np.float64)
+    for t in range(n_tokens):
+        raw_rows, comp_rows = indexed_visit_rows(
+            raw_cap=raw.shape[0], n_comp=comp.shape[0], topk=np.asarray(topk)[t], qpos=int(pos0) + t,
+            last_pos=last_pos, window=int(window), ratio=int(ratio), raw_start=int(raw_start))
+        rows = np.concatenate([raw[raw_rows].reshape(-1, raw.shape[1]),
+                               comp[comp_rows].reshape(-1, raw.shape[1])], axis=0)
+        out[t] = attend_rows_f64(round_f16(q[t].astype(F32)), rows, sinks, float(q.shape[-1]) ** -0.5)
+    return out
+
+
+# --------------------------------------------------------------------------
+# a6/a9: fused decode island
+# --------------------------------------------------------------------------
+
+def prepared_kv_row(kv_row_f16: np.ndarray, pos: int, inv_freq: np.ndarray) -> np.ndarray:
+    """Rope tail + FP8 prefix round trip of the new KV row, float16 bits.
+
+    decode_attention_kernel.py:223-262: dims < 448 take the FP8 round trip of
+    the float16 values widened to float32, rounded back to float16; dims >=
+    448 take the partial rope at float16 op rounding from the pre-rope values.
+    """
+    row = np.asarray(kv_row_f16, dtype=np.float16).astype(F32).reshape(512)
+    rt = fp8_kv_roundtrip(row.reshape(1, 512)).reshape(512)
+    roped = partial_rope_lowp(row.reshape(1, 512), pos, inv_freq).reshape(512)
+    out = np.concatenate([rt[:448], roped[448:]])
+    with np.errstate(over="ignore"):
+        return out.astype(np.float16)
+
+
+def fused_decode_prep(q_idx, pooled_qat, weights, kv_row, inv_freq, params, *, scale: float, topk: int):
+    """a6: scores (float64 from half-staged QAT q), radix top-k, prepared KV row.
+
+    decode_attention_kernel.py:194-376. The top-k is taken on the float32
+    rounding of the float64 scores; a device that accumulates in another order
+    is compared on its own scores (see tests).
+    """
+    q = np.asarray(q_idx)
+    qq = round_f16(indexer_qat(q.astype(F32)))
+    scores = indexer_scores_f64(qq, pooled_qat, weights, scale)
+    sel = radix_select_topk(scores.astype(F32), topk)
+    row = prepared_kv_row(kv_row, int(np.asarray(params).reshape(-1)[0]), inv_freq)
+    return sel, row, scores
+
+
+def fused_decode_sdpa(q, window, row, pooled, sel, sinks, inv_freq, params, *, scale: float) -> np.ndarray:
+    """a9: rope(q) -> softmax over window(with row substituted) + pooled[sel] + sink -> f16 -> inverse rope.
+
+    decode_attention_kernel.py:381-522. Returns float16 ``[H,512]``.
+    """
+    p = np.asarray(params).reshape(-1)
+    pos, write_idx = int(p[0]), int(p[1])
+    qh = partial_rope_lowp(np.asarray(q, dtype=np.float16).astype(F32), pos, inv_freq)
+    win = np.asarray(window, dtype=np.float16).astype(F32).copy()
+    if 0 <= write_idx < win.shape[0]:
+        win[write_idx] = np.asarray(row, dtype=np.float16).astype(F32)
+    pool = np.asarray(pooled, dtype=np.float16).astype(F32)
+    keys = np.concatenate([win, pool[np.asarray(sel, dtype=np.int64)]], axis=0)
+    out = attend_rows_f64(qh, keys, np.asarray(sinks, dtype=np.float16).astype(np.float64), scale)
+    out_h = round_f16(out.astype(F32))
+    out_h = partial_rope_lowp(out_h, pos, inv_freq, inverse=True)
+    return out_h.astype(np.float16)
+
+
+# --------------------------------------------------------------------------
+# BASELINE config 4/5 shapes (batched extensions of a3/a6/a8)
+# --------------------------------------------------------------------------
+
+def e4m3_decode(codes: np.ndarray) -> np.ndarray:
+    """Decode E4M3FN bytes to float32 (0x7F/0xFF = NaN)."""
+    c = np.asarray(codes, dtype=np.uint8)
+    mag = c & 0x7F
+    table = np.concatenate([e4m3fn_values(), np.asarray([np.nan], dtype=F32)])
+    v = table[mag.astype(np.int64)]
+    return np.where(c & 0x80, -v, v).astype(F32)
+
+
+def e4m3_encode(x: np.ndarray) -> np.ndarray:
+    """Encode float32 to E4M3FN bytes, nearest, ties to even code, saturating at 448."""
+    x = np.asarray(x, dtype=F32)
+    table = e4m3fn_values().astype(np.float64)
+    a = np.minimum(np.abs(x).astype(np.float64), 448.0)
+    hi = np.searchsorted(table, a, side="left").clip(0, 126)
+    lo = (hi - 1).clip(0, 126)
+    dlo = np.abs(a - table[lo])
+    dhi = np.abs(table[hi] - a)
+    pick_hi = (dhi < dlo) | ((dhi == dlo) & (hi % 2 == 0))
+    code = np.where(pick_hi, hi, lo).astype(np.uint8)
+    return np.where(np.signbit(x), code | 0x80, code).astype(np.uint8)
+
+
+def indexer_scores_fp8(q: np.ndarray, key_codes: np.ndarray, key_scales: np.ndarray,
+                       weights: np.ndarray) -> np.ndarray:
+    """Lightning-indexer score row with FP8 keys, float64.
+
+    ``score[b,r] = sum_h w[b,h] * relu(q[b,h] . (e4m3(codes[b,r]) * kscale[b,r]))``;
+    the batched, fp8-key form of a3 named by BASELINE config 4.
+    q ``[B,H,128]`` (bf16 values as float32), key_codes uint8 ``[B,N,128]``,
+    key_scales f32 ``[B,N]``, weights f32 ``[B,H]`` -> ``[B,N]``.
+    """
+    q = np.asarray(q, dtype=np.float64)
+    k = e4m3_decode(key_codes).astype(np.float64) * np.asarray(key_scales, dtype=np.float64)[..., None]
+    w = np.asarray(weights, dtype=np.float64)
+    raw = np.einsum("bhd,bnd->bhn", q, k)
+    return np.einsum("bhn,bh->bn", np.maximum(raw, 0.0), w)
+
+
+def sparse_mla_decode(q: np.ndarray, kv: np.ndarray, rows: np.ndarray, *, scale: float, v_dim: int = 512,
+                      sinks=None) -> np.ndarray:
+    """Gathered multi-head latent decode attention, float64 (batched form of a8).
+
+    q ``[B,H,Dk]``, kv ``[B,N,Dk]`` (V = first ``v_dim`` dims of each row),
+    rows int ``[B,R]`` gathered row ids (negative = skipped) -> ``[B,H,v_dim]``.
+    """
+    q = np.asarray(q, dtype=np.float64)
+    rows = np.asarray(rows, dtype=np.int64)
+    out = np.zeros((q.shape[0], q.shape[1], v_dim), dtype=np.float64)
+    for b in range(q.shape[0]):
+        r = rows[b]
+        r = r[r >= 0]
+        k = np.asarray(kv[b][r], dtype=np.float64)
+        out[b] = attend_rows_f64(q[b], k, None if sinks is None else sinks, scale, v_dim=v_dim)
+    return out
