@@ -45,7 +45,8 @@ def test_affine_q8_round_trip_and_packing():
     deq = qwen.affine_q8_dequantize(packed, scales, biases)
     span = (x.reshape(3, 5, 4, 64).max(-1) - x.reshape(3, 5, 4, 64).min(-1))
     err = np.abs(deq - x).reshape(3, 5, 4, 64).max(-1)
-    assert np.all(err <= span / 255.0 * 0.5 + 1e-6)
+    # the rescaled step (edge / round(edge/scale)) lets the far edge clip by < one step
+    assert np.all(err <= span / 255.0 + 1e-6)
     # element j of each word lives in bits [8j, 8j+8)
     codes = np.clip(np.rint((x.reshape(3, 5, 4, 64) - biases[..., None]) / scales[..., None]), 0, 255)
     codes = codes.reshape(3, 5, 256).astype(np.uint32)
