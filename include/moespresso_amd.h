@@ -1,0 +1,147 @@
+/*
+ * C-ABI of libmoespresso_amd.so: hand-written gfx950 (MI355X) kernels for the
+ * MoEspresso attention hot path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host";
+ *   - tensors are dense row-major with the shapes given, no strides;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); the
+ *     call only enqueues work, it never synchronises and never allocates;
+ *   - scratch memory is passed in by the caller (`workspace`), its size comes
+ *     from the matching *_workspace_bytes function;
+ *   - return value 0 = enqueued; MSPR_ERR_ARG = rejected before any launch
+ *     (shape / dtype / alignment / workspace too small); MSPR_ERR_LAUNCH = HIP
+ *     reported a launch error. mspr_last_error() gives the reason as text.
+ *
+ * Each entry point cites the reference interface it stands in for (paths under
+ * the reference tree). Entry points marked "extension" have the BASELINE
+ * configuration shapes (batch > 1, fp8 keys, 576/512 MLA, bf16, g32 Q8) that
+ * the reference's own callables reject.
+ */
+#ifndef MOESPRESSO_AMD_H
+#define MOESPRESSO_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSPR_OK 0
+#define MSPR_ERR_ARG (-1)
+#define MSPR_ERR_LAUNCH (-2)
+
+/* element type codes */
+#define MSPR_F32 0
+#define MSPR_F16 1
+#define MSPR_BF16 2
+
+/* Library ABI version (bumped on any signature change). */
+int mspr_abi_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* mspr_last_error(void);
+
+/* ------------------------------------------------------------------ DS4 indexer */
+
+/* Hadamard-128 + e2m1 activation round trip over 128-wide rows, float32 out.
+ * Replaces indexer_qat_rows, src/moespresso/runtime/deepseek_v4/indexer_score_kernel.py:284
+ * (= _dsv4_indexer_qat, model.py:745). x: [n_rows,128] of x_dtype; out: f32 [n_rows,128]. */
+int mspr_indexer_qat_rows(const void* x, int x_dtype, int64_t n_rows, float* out, void* stream);
+
+/* Decode score row with the query QAT applied in-kernel:
+ *   scores[r] = sum_h max(qat(q_h) . pooled[r], 0) * scale * weights[h]
+ * Replaces fused_qat_indexer_scores, indexer_score_kernel.py:354.
+ * q: [n_heads,128] of q_dtype (1..64 heads); pooled_qat: f32 [n_rows,128];
+ * weights: f32 [n_heads]; scores: f32 [n_rows]. */
+int mspr_fused_qat_indexer_scores(const void* q, int q_dtype, int n_heads, const float* pooled_qat,
+                                  int64_t n_rows, const float* weights, float scale, float* scores,
+                                  void* stream);
+
+/* relu, score scale, head-weight cast and n_heads^-1/2 scale, head sum, capacity pad, negate.
+ * Replaces fused_score_tail, indexer_score_kernel.py:562.
+ * scores: f32 [n_heads,capacity] (32..64 heads); weights_raw: [n_heads] of w_dtype;
+ * params: int32 [>=2], params[1] = valid columns; neg: f32 [capacity]. */
+int mspr_indexer_score_tail(const float* scores, int n_heads, int64_t capacity, const void* weights_raw,
+                            int w_dtype, const int32_t* params, float scale, float* neg, void* stream);
+
+/* E4M3FN round trip of dims [0,448) in 64-blocks of 512-wide float32 rows, tail copied.
+ * Replaces fp8_kv_prefix_rows, decode_attention_kernel.py:587
+ * (= _deepseek_v4_fp8_kv_roundtrip, model.py:559). x/out: f32 [n_rows,512]. */
+int mspr_fp8_kv_prefix_rows(const float* x, int64_t n_rows, float* out, void* stream);
+
+/* Deterministic top-k over float32 score rows: rows whose monotone key is strictly above the
+ * k-th value in ascending row order, then the lowest-index rows tied with it.
+ * Stands in for mx.argpartition(-scores, kth=k-1)[..., :k] (model.py:1003,1057,1443) with the
+ * emission order of the prep kernel's phase C, decode_attention_kernel.py:295-375.
+ * scores: f32 [batch,n_rows] (row b at scores + b*score_stride); sel: int32 [batch,topk];
+ * 0 < topk <= n_rows. No 16-bit row limit. */
+int mspr_topk_select(const float* scores, int64_t score_stride, int batch, int64_t n_rows, int topk,
+                     int32_t* sel, void* stream);
+
+/* One ratio-4 decode token: in-kernel query QAT (staged as float16), score row, deterministic
+ * top-k, and the prepared KV row (rope tail + E4M3FN prefix round trip).
+ * Replaces fused_decode_prep, decode_attention_kernel.py:669.
+ * q_idx: [n_heads,128] of q_dtype; pooled_qat: f32 [n_rows,128]; weights: f32 [n_heads];
+ * kv_row: f16 [512]; inv_freq: f32 [32]; params: int32, params[0] = position;
+ * outputs sel: int32 [topk], row_out: f16 [512], scores: f32 [n_rows]. 0 < topk < n_rows. */
+int mspr_fused_decode_prep(const void* q_idx, int q_dtype, int n_heads, const float* pooled_qat,
+                           int64_t n_rows, const float* weights, const void* kv_row,
+                           const float* inv_freq, const int32_t* params, float scale, int topk,
+                           int32_t* sel, void* row_out, float* scores, void* stream);
+
+/* Extension (BASELINE config 4): batched lightning-indexer scores with FP8 keys.
+ *   scores[b,r] = sum_h w[b,h] * relu(q[b,h] . e4m3(keys[b,r])) * key_scales[b,r]
+ * q: bf16 [batch,n_heads,128] (n_heads <= 64); keys: E4M3FN bytes [batch,n_rows,128];
+ * key_scales: f32 [batch,n_rows] (> 0); weights: f32 [batch,n_heads]; scores: f32 [batch,n_rows]. */
+int mspr_indexer_scores_fp8(const void* q, const void* keys, const float* key_scales,
+                            const float* weights, int batch, int n_heads, int64_t n_rows,
+                            float* scores, void* stream);
+
+/* ------------------------------------------------------------------ DS4 sparse attention */
+
+/* Scratch bytes for the three gathered-attention entry points below. */
+size_t mspr_sparse_attention_workspace_bytes(int batch, int n_heads, int64_t n_keys);
+
+/* One-token indexed mixed attention over a ring of raw rows plus gathered pool rows, K == V.
+ * Replaces indexed_mixed_attention_decode, indexed_attention_kernel.py:1496 (kernel :61-174).
+ * q: f32 [n_heads,512] (rounded to half on load); raw_kv: f16 [raw_cap,512];
+ * comp_kv: f16 [n_comp,512]; topk: int32 [top_k]; sinks: f32 [n_heads]; out: f32 [n_heads,512].
+ * Ids < 0 are skipped; the first id >= min((pos0+1)/ratio, n_comp) ends the walk
+ * (ratio 0 = whole pool visible). */
+int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, const void* raw_kv, int raw_cap,
+                                        const void* comp_kv, int64_t n_comp, const int32_t* topk,
+                                        int top_k, const float* sinks, int64_t pos0, int window,
+                                        int ratio, int raw_start, float* out, void* workspace,
+                                        size_t workspace_bytes, void* stream);
+
+/* Decode SDPA of the fused island: rope(q), softmax over the window (row substituted at
+ * params[1]) + pooled[sel] + per-head sink, float16 output, inverse rope.
+ * Replaces fused_decode_sdpa, decode_attention_kernel.py:733.
+ * q: f16 [n_heads,512]; window: f16 [window_rows,512]; row: f16 [512]; pooled: f16 [n_rows,512];
+ * sel: int32 [n_sel]; sinks: f16 [n_heads]; inv_freq: f32 [32]; params: int32 [position, write_idx];
+ * out: f16 [n_heads,512]. */
+int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* window, int window_rows,
+                           const void* row, const void* pooled, int64_t n_rows, const int32_t* sel,
+                           int n_sel, const void* sinks, const float* inv_freq, const int32_t* params,
+                           float scale, void* out, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/* Extension (BASELINE config 5): batched sparse multi-head latent decode attention.
+ * Every head of batch b attends rows kv[b, rows[b, :]] of a shared latent cache; K is the whole
+ * k_dim-wide row and V its first v_dim columns.
+ * q: [batch,n_heads,k_dim] of dtype (f16|bf16); kv: [batch,n_pool,k_dim] same dtype;
+ * rows: int32 [batch,n_rows] gathered ids (negative or >= n_pool = skipped); the contiguous
+ * window kv[b, win_start : win_start+win_rows] is attended as well (win_rows may be 0);
+ * sinks: f32 [n_heads] or NULL; out: [batch,n_heads,v_dim] same dtype.
+ * k_dim in {512,576}, v_dim = 512, n_heads <= 128. */
+int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, const float* sinks,
+                           int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
+                           int n_rows, int64_t win_start, int win_rows, float scale, void* out,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOESPRESSO_AMD_H */

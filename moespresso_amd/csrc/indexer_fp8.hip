@@ -1,0 +1,136 @@
+// Batched lightning-indexer score row with FP8 (E4M3FN) keys and one float32 scale per key:
+//   score[b, r] = sum_h w[b, h] * relu(q[b, h] . e4m3(keys[b, r])) * key_scale[b, r]
+//
+// The 64-head x 128-wide contraction against each key runs on the bf16 MFMA (32x32x16): heads
+// are the M dimension, keys the N dimension, so the relu-weighted head sum of one key stays in one
+// lane's accumulator registers (plus one xor-32 shuffle). E4M3 values are exact in bf16, and a
+// bf16 x bf16 product is exact in the float32 accumulator, so the only rounding is the
+// accumulation itself. Keys stream from HBM straight into the B-operand registers: a lane owns
+// 64 contiguous bytes of its key row, a wave 4 KB of contiguous memory per 32-key tile, and the
+// next tile is in flight while the current one is multiplied.
+#include "common.h"
+
+namespace {
+
+// Two E4M3FN bytes (the low or high half of `w`) to two bf16 values packed in one register.
+__device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
+  f32x2_t f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+  // bf16 = top 16 bits of the float32 (exact: E4M3 carries 3 mantissa bits)
+  return __builtin_amdgcn_perm(__float_as_uint(f.y), __float_as_uint(f.x), 0x07060302u);
+}
+
+__global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16_t* __restrict__ q,
+                                                                    const uint8_t* __restrict__ keys,
+                                                                    const float* __restrict__ key_scales,
+                                                                    const float* __restrict__ weights, int n_heads,
+                                                                    int64_t n_rows, int blocks_per_batch,
+                                                                    float* __restrict__ scores) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int m = lane & 31;
+  const int g = lane >> 5;
+  const int b = blockIdx.x / blocks_per_batch;
+  const int blk = blockIdx.x % blocks_per_batch;
+
+  const uint16_t* qb = q + (int64_t)b * n_heads * 128;
+  const uint8_t* kb = keys + (int64_t)b * n_rows * 128;
+  const float* ksb = key_scales + (int64_t)b * n_rows;
+  const float* wb = weights + (int64_t)b * n_heads;
+  float* sb = scores + (int64_t)b * n_rows;
+
+  // A operand: lane (m -> head, g) holds q[head][64g + 8s .. +7] for k-step s; heads past the end are zero
+  u32x4_t qa[2][8];
+#pragma unroll
+  for (int mt = 0; mt < 2; mt++) {
+    const int head = 32 * mt + m;
+    const bool live = head < n_heads;
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(qb + (int64_t)(live ? head : 0) * 128 + 64 * g);
+#pragma unroll
+    for (int s = 0; s < 8; s++) qa[mt][s] = live ? p[s] : u32x4_t{0u, 0u, 0u, 0u};
+  }
+  // weights of this lane's accumulator rows: head = 32mt + 8(i/4) + 4g + i%4
+  float wl[2][16];
+#pragma unroll
+  for (int mt = 0; mt < 2; mt++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int head = 32 * mt + 8 * (i / 4) + 4 * g + (i % 4);
+      wl[mt][i] = head < n_heads ? wb[head] : 0.0f;
+    }
+
+  const int64_t n_tiles = (n_rows + 31) / 32;
+  const int64_t stride = (int64_t)blocks_per_batch * 4;
+  int64_t tile = (int64_t)blk * 4 + wave;
+  if (tile >= n_tiles) return;
+
+  auto load_tile = [&](int64_t t, u32x4_t (&raw)[4]) {
+    int64_t row = t * 32 + m;
+    if (row >= n_rows) row = n_rows - 1;
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(kb + row * 128 + 64 * g);
+#pragma unroll
+    for (int j = 0; j < 4; j++) raw[j] = p[j];
+  };
+
+  u32x4_t cur[4], nxt[4];
+  load_tile(tile, cur);
+  for (; tile < n_tiles; tile += stride) {
+    const bool more = tile + stride < n_tiles;
+    if (more) load_tile(tile + stride, nxt);
+    const int64_t row = tile * 32 + m;
+    const float ks = ksb[row < n_rows ? row : n_rows - 1];
+
+    f32x16_t acc0 = {0}, acc1 = {0};
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      // bytes 8s..8s+7 of this lane's 64: two dwords of cur[s/2]
+      const uint32_t w0 = cur[s >> 1][(s & 1) * 2], w1 = cur[s >> 1][(s & 1) * 2 + 1];
+      u32x4_t kf = {fp8x2_to_bf16x2(w0, false), fp8x2_to_bf16x2(w0, true), fp8x2_to_bf16x2(w1, false),
+                    fp8x2_to_bf16x2(w1, true)};
+      bf16x8_t kfb = __builtin_bit_cast(bf16x8_t, kf);
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, qa[0][s]), kfb, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, qa[1][s]), kfb, acc1, 0, 0, 0);
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) sum = fmaf(fmaxf(acc0[i], 0.0f), wl[0][i], sum);
+#pragma unroll
+    for (int i = 0; i < 16; i++) sum = fmaf(fmaxf(acc1[i], 0.0f), wl[1][i], sum);
+    sum += __shfl_xor(sum, 32, MSPR_WAVE);
+    if (g == 0 && row < n_rows) sb[row] = sum * ks;
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) cur[j] = nxt[j];
+    }
+  }
+}
+
+}  // namespace
+
+int mspr_launch_indexer_scores_fp8(const void* q, const void* keys, const float* key_scales, const float* weights,
+                                   int batch, int n_heads, int64_t n_rows, float* scores, hipStream_t st) {
+  const int64_t n_tiles = (n_rows + 31) / 32;
+  // about 2 workgroups per CU in total, every wave with at least one tile
+  int64_t per_batch = (512 + batch - 1) / batch;
+  int64_t max_blocks = (n_tiles + 3) / 4;
+  if (per_batch > max_blocks) per_batch = max_blocks;
+  if (per_batch < 1) per_batch = 1;
+  dim3 grid((unsigned)(per_batch * batch)), block(256);
+  indexer_scores_fp8_kernel<<<grid, block, 0, st>>>(reinterpret_cast<const uint16_t*>(q),
+                                                     reinterpret_cast<const uint8_t*>(keys), key_scales, weights,
+                                                     n_heads, n_rows, (int)per_batch, scores);
+  MSPR_CHECK_LAUNCH("indexer_scores_fp8");
+  return MSPR_OK;
+}
+
+extern "C" int mspr_indexer_scores_fp8(const void* q, const void* keys, const float* key_scales,
+                                       const float* weights, int batch, int n_heads, int64_t n_rows, float* scores,
+                                       void* stream) {
+  MSPR_REQUIRE(q && keys && key_scales && weights && scores, "indexer_scores_fp8: null pointer");
+  MSPR_REQUIRE(batch >= 1, "indexer_scores_fp8: batch must be positive");
+  MSPR_REQUIRE(n_heads >= 1 && n_heads <= 64, "indexer_scores_fp8: between 1 and 64 heads");
+  MSPR_REQUIRE(n_rows >= 1 && n_rows < ((int64_t)1 << 31), "indexer_scores_fp8: n_rows out of range");
+  MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(keys, 16), "indexer_scores_fp8: q and keys must be 16-byte aligned");
+  return mspr_launch_indexer_scores_fp8(q, keys, key_scales, weights, batch, n_heads, n_rows, scores,
+                                        (hipStream_t)stream);
+}

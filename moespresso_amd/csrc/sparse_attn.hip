@@ -1,0 +1,671 @@
+// Gathered ("indexed") decode attention over a latent KV cache shared by all heads.
+//
+// One query token per batch entry attends a list of key slots: first a window segment (a ring of
+// raw rows, optionally with one slot replaced by a freshly prepared row), then rows gathered from
+// a pool by index. K is the whole row (512 or 576 wide), V its first 512 columns.
+//
+// Work split: a workgroup owns (batch, 64-head block, slot range) and streams 32-slot tiles.
+// Each K row is read from HBM once and staged row-major in LDS (double buffered). The four waves
+// are (head group hg of 32 heads) x (half dh): for S^T = K.Q^T a wave contracts its half of the
+// row width and the two halves are summed through LDS; for O^T = V^T.P^T it owns 256 of the 512
+// output columns. V^T operands come out of the same row-major tile through the LDS transpose
+// read, so no second copy of the tile exists. Partial (m, l, O) per slot range are merged by a
+// second kernel (log-sum-exp), which also applies the sink, the normalisation, the output cast
+// and the optional inverse rope.
+//
+// MFMA shapes: v_mfma_f32_32x32x16_{f16,bf16}. Accumulator layout (lane l, register i):
+// column = l % 32, row = 8*(i/4) + 4*(l/32) + i%4. In S^T the column is the head and the row the
+// key, so softmax statistics are per lane; P^T registers feed the next MFMA's B operand unchanged.
+#include "common.h"
+
+namespace {
+
+constexpr int kTile = 32;
+constexpr int kDV = 512;
+constexpr int kThreads = 256;
+
+struct SparseAttnArgs {
+  // query
+  const void* q;
+  int q_dtype;
+  int64_t q_batch_stride;  // elements
+  int n_heads;
+  int batch;
+  // window segment
+  const void* win;
+  int64_t win_batch_stride;
+  int n_win;
+  int win_first;  // logical index of the first visited ring row
+  int raw_start;
+  int raw_cap;
+  const void* subst_row;
+  int subst_slot;          // window slot replaced by subst_row (-1: none)
+  int subst_from_params;   // take the slot from params[1] on the device instead
+  // gathered segment
+  const void* pool;
+  int64_t pool_batch_stride;
+  int64_t n_pool;
+  const int32_t* idx;
+  int64_t idx_batch_stride;
+  int n_idx;
+  int64_t visible;  // ids >= visible end the walk
+  int check_stop;
+  // softmax
+  const void* sinks;
+  int sinks_dtype;
+  float scale_log2;
+  // rope
+  const float* inv_freq;
+  const int32_t* params;
+  int rope;
+  // split
+  int n_splits;
+  int slots_per_split;
+  int n_hblk;
+  float* ws_o;
+  float* ws_ml;
+  // output
+  void* out;
+  int out_dtype;
+};
+
+template <int KDT>
+__device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
+  if constexpr (KDT == MSPR_BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
+                                                   c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c,
+                                                  0, 0, 0);
+  }
+}
+
+template <int KDT>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  if constexpr (KDT == MSPR_BF16) {
+    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+  } else {
+    return (uint32_t)f32_to_f16_bits(a) | ((uint32_t)f32_to_f16_bits(b) << 16);
+  }
+}
+
+template <int KDT>
+__device__ __forceinline__ float unpack_lo(uint32_t w) {
+  if constexpr (KDT == MSPR_BF16) return bf16_bits_to_f32((uint16_t)(w & 0xFFFFu));
+  else return f16_bits_to_f32((uint16_t)(w & 0xFFFFu));
+}
+template <int KDT>
+__device__ __forceinline__ float unpack_hi(uint32_t w) {
+  if constexpr (KDT == MSPR_BF16) return bf16_bits_to_f32((uint16_t)(w >> 16));
+  else return f16_bits_to_f32((uint16_t)(w >> 16));
+}
+
+template <int KDT>
+__device__ __forceinline__ float round_to_kdt(float v) {
+  if constexpr (KDT == MSPR_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  else return f16_bits_to_f32(f32_to_f16_bits(v));
+}
+
+// Eight consecutive query elements as one packed operand register group, converted to the KV type.
+template <int KDT>
+__device__ __forceinline__ void load_q8(const void* q, int q_dtype, int64_t off, float (&v)[8]) {
+  if (q_dtype == MSPR_F32) {
+    const f32x4_t* p = reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(q) + off);
+    f32x4_t a = p[0], b = p[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+    u32x4_t w = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(q) + off);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      if (q_dtype == MSPR_F16) {
+        v[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xFFFFu));
+        v[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+      } else {
+        v[2 * j] = bf16_bits_to_f32((uint16_t)(w[j] & 0xFFFFu));
+        v[2 * j + 1] = bf16_bits_to_f32((uint16_t)(w[j] >> 16));
+      }
+    }
+  }
+}
+
+template <int DK>
+struct Geometry {
+  static constexpr int kChunks = DK / 8;          // 16-byte chunks per row
+  static constexpr int kLoads = kChunks / 8;      // per loader thread (8 threads per row)
+  static constexpr int kPitch = DK * 2 + 16;      // bytes; +16 keeps 8 consecutive rows on distinct 16B bank groups
+  static constexpr int kHalf = DK / 2;            // contraction columns per dh wave
+  static constexpr int kSteps = kHalf / 16;       // MFMA k-steps per dh wave
+  static constexpr int kTileBytes = kTile * kPitch;
+  static constexpr int kSxBytes = 4 * 16 * 64 * 4;  // 4 waves x 16 floats x 64 lanes
+  static constexpr int kLdsBytes = 2 * kTileBytes + 2 * kSxBytes + 2 * 32 * 4 + 2 * 4 + 16;
+};
+
+template <int KDT, int DK>
+__global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAttnArgs a) {
+  using G = Geometry<DK>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  unsigned char* kbuf = lds;                                       // [2][kTile][kPitch]
+  float* sx = reinterpret_cast<float*>(lds + 2 * G::kTileBytes);   // [2][4][16*64]
+  float* rope_c = reinterpret_cast<float*>(lds + 2 * G::kTileBytes + 2 * G::kSxBytes);
+  float* rope_s = rope_c + 32;
+  uint8_t* vmask = reinterpret_cast<uint8_t*>(rope_s + 32);        // [2][4] one byte per wave per buffer
+  int* stop_shared = reinterpret_cast<int*>(vmask + 8);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int hg = wave >> 1;
+  const int dh = wave & 1;
+  const int n = lane & 31;  // MFMA column: head (S^T, O^T); MFMA row for A operands
+  const int g = lane >> 5;
+
+  // ---- workgroup -> (batch, head block, split); consecutive splits of one batch share an XCD
+  const int total = gridDim.x;
+  int work = blockIdx.x;
+  if ((total & 7) == 0) work = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+  const int sp = work % a.n_splits;
+  const int bh = work / a.n_splits;
+  const int hb = bh % a.n_hblk;
+  const int b = bh / a.n_hblk;
+
+  const int n_keys = a.n_win + a.n_idx;
+  const int slot0 = sp * a.slots_per_split;
+  int slot1 = slot0 + a.slots_per_split;
+  if (slot1 > n_keys) slot1 = n_keys;
+  const int n_tiles = slot1 > slot0 ? (slot1 - slot0 + kTile - 1) / kTile : 0;
+
+  const uint16_t* win_b = reinterpret_cast<const uint16_t*>(a.win) + (int64_t)b * a.win_batch_stride;
+  const uint16_t* pool_b = reinterpret_cast<const uint16_t*>(a.pool) + (int64_t)b * a.pool_batch_stride;
+  const int32_t* idx_b = a.idx + (int64_t)b * a.idx_batch_stride;
+
+  // ---- prologue: stop position of the gathered walk, rope table
+  if (tid == 0) *stop_shared = a.n_idx;
+  if (a.rope && tid < 32) {
+    float theta = (float)a.params[0] * a.inv_freq[tid];
+    rope_c[tid] = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
+    rope_s[tid] = f16_bits_to_f32(f32_to_f16_bits((float)sin((double)theta)));
+  }
+  __syncthreads();
+  if (a.check_stop) {
+    int first = a.n_idx;
+    for (int i = tid; i < a.n_idx; i += kThreads) {
+      int id = idx_b[i];
+      if (id >= 0 && (int64_t)id >= a.visible && i < first) first = i;
+    }
+    if (first < a.n_idx) atomicMin(stop_shared, first);
+    __syncthreads();
+  }
+  const int stop_pos = *stop_shared;
+  const int subst_slot = a.subst_from_params ? a.params[1] : a.subst_slot;
+
+  // ---- loader role: thread owns row r of the tile and chunks sub, sub+8, ...
+  const int lrow = tid >> 3;
+  const int lsub = tid & 7;
+  auto slot_src = [&](int slot) -> const uint16_t* {
+    if (slot >= slot1) return nullptr;
+    if (slot < a.n_win) {
+      if (slot == subst_slot) return reinterpret_cast<const uint16_t*>(a.subst_row);
+      int r = (int)(((int64_t)a.raw_start + a.win_first + slot) % a.raw_cap);
+      return win_b + (int64_t)r * DK;
+    }
+    int i = slot - a.n_win;
+    if (i >= stop_pos) return nullptr;
+    int id = idx_b[i];
+    if (id < 0 || (int64_t)id >= a.n_pool) return nullptr;
+    return pool_b + (int64_t)id * DK;
+  };
+  u32x4_t stage[G::kLoads];
+  bool stage_valid = false;
+  auto issue_loads = [&](int tile) {
+    const uint16_t* src = slot_src(slot0 + tile * kTile + lrow);
+    stage_valid = src != nullptr;
+    if (stage_valid) {
+      const u32x4_t* p = reinterpret_cast<const u32x4_t*>(src);
+#pragma unroll
+      for (int j = 0; j < G::kLoads; j++) stage[j] = p[lsub + 8 * j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < G::kLoads; j++) stage[j] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+  };
+  auto store_stage = [&](int buf) {
+    unsigned char* dst = kbuf + buf * G::kTileBytes + lrow * G::kPitch;
+#pragma unroll
+    for (int j = 0; j < G::kLoads; j++) *reinterpret_cast<u32x4_t*>(dst + (lsub + 8 * j) * 16) = stage[j];
+    // one validity byte per wave: bit j = row 8*wave + j
+    uint64_t bal = __ballot(stage_valid);
+    if (lane == 0) {
+      uint32_t byte = 0u;
+#pragma unroll
+      for (int j = 0; j < 8; j++) byte |= (uint32_t)((bal >> (8 * j)) & 1ull) << j;
+      vmask[buf * 4 + wave] = (uint8_t)byte;
+    }
+  };
+
+  if (n_tiles > 0) issue_loads(0);
+
+  // ---- query operand: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7] per k-step
+  const int head = hb * 64 + hg * 32 + n;
+  u32x4_t qf[G::kSteps];
+  {
+    const bool live = head < a.n_heads;
+    const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)(live ? head : 0) * DK;
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) {
+      const int d0 = dh * G::kHalf + 16 * ks + 8 * g;
+      float v[8];
+      load_q8<KDT>(a.q, a.q_dtype, qoff + d0, v);
+#pragma unroll
+      for (int j = 0; j < 8; j++) v[j] = live ? round_to_kdt<KDT>(v[j]) : 0.0f;
+      if (a.rope && d0 >= DK - 64) {
+        // partial rope on interleaved pairs with every product and sum rounded to the element type
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          int p = (d0 - (DK - 64)) / 2 + j;
+          float c = rope_c[p], s = rope_s[p];
+          float x0 = v[2 * j], x1 = v[2 * j + 1];
+          float m0 = round_to_kdt<KDT>(x0 * c), m1 = round_to_kdt<KDT>(x1 * s);
+          float m2 = round_to_kdt<KDT>(x0 * s), m3 = round_to_kdt<KDT>(x1 * c);
+          v[2 * j] = round_to_kdt<KDT>(m0 - m1);
+          v[2 * j + 1] = round_to_kdt<KDT>(m2 + m3);
+        }
+      }
+      qf[ks] = u32x4_t{pack2<KDT>(v[0], v[1]), pack2<KDT>(v[2], v[3]), pack2<KDT>(v[4], v[5]), pack2<KDT>(v[6], v[7])};
+    }
+  }
+
+  f32x16_t oacc[8];
+#pragma unroll
+  for (int mt = 0; mt < 8; mt++) oacc[mt] = f32x16_t{0};
+  float m_run = -__builtin_inff();
+  float l_run = 0.0f;
+
+  if (n_tiles > 0) store_stage(0);
+  __syncthreads();
+
+  // per-lane LDS offsets
+  const int a_row_off = n * G::kPitch + (dh * G::kHalf + 8 * g) * 2;                     // QK^T A operand
+  const int tr_s = lane & 15;
+  const int tr_off = (4 * g + (tr_s >> 2)) * G::kPitch + (dh * 256 + 16 * ((lane >> 4) & 1) + 4 * (tr_s & 3)) * 2;
+
+  for (int t = 0; t < n_tiles; t++) {
+    const int buf = t & 1;
+    if (t + 1 < n_tiles) issue_loads(t + 1);
+    const unsigned char* kt = kbuf + buf * G::kTileBytes;
+
+    // S^T partial over this wave's half of the row width
+    f32x16_t sacc = {0};
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) {
+      u32x4_t af = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + ks * 32);
+      sacc = mfma32<KDT>(af, qf[ks], sacc);
+    }
+    float* sxw = sx + (buf * 4 + wave) * (16 * 64);
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+      *reinterpret_cast<f32x4_t*>(sxw + (c * 64 + lane) * 4) =
+          f32x4_t{sacc[4 * c], sacc[4 * c + 1], sacc[4 * c + 2], sacc[4 * c + 3]};
+    __syncthreads();
+    const float* sxp = sx + (buf * 4 + (wave ^ 1)) * (16 * 64);
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      f32x4_t o = *reinterpret_cast<const f32x4_t*>(sxp + (c * 64 + lane) * 4);
+      sacc[4 * c] += o.x;
+      sacc[4 * c + 1] += o.y;
+      sacc[4 * c + 2] += o.z;
+      sacc[4 * c + 3] += o.w;
+    }
+
+    // online softmax in the log2 domain; key of register i is 8*(i/4) + 4g + i%4
+    const uint32_t mask = *reinterpret_cast<const uint32_t*>(vmask + buf * 4) >> (4 * g);
+    float tmax = -__builtin_inff();
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const bool valid = (mask >> (8 * (i / 4) + (i % 4))) & 1u;
+      float s = valid ? sacc[i] * a.scale_log2 : -__builtin_inff();
+      sacc[i] = s;
+      tmax = fmaxf(tmax, s);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, MSPR_WAVE));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_safe = m_new == -__builtin_inff() ? 0.0f : m_new;
+    const float alpha = exp2f(m_run - m_safe);
+    float psum = 0.0f;
+    float p[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      p[i] = exp2f(sacc[i] - m_safe);
+      psum += p[i];
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (!__all(alpha == 1.0f)) {
+#pragma unroll
+      for (int mt = 0; mt < 8; mt++) oacc[mt] = oacc[mt] * alpha;
+    }
+    u32x4_t pf[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+      pf[ks] = u32x4_t{pack2<KDT>(p[8 * ks], p[8 * ks + 1]), pack2<KDT>(p[8 * ks + 2], p[8 * ks + 3]),
+                       pack2<KDT>(p[8 * ks + 4], p[8 * ks + 5]), pack2<KDT>(p[8 * ks + 6], p[8 * ks + 7])};
+
+    // O^T += V^T . P^T ; V^T operands through the LDS transpose read of the row-major tile
+#pragma unroll
+    for (int mt = 0; mt < 8; mt++) {
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        const unsigned char* base = kt + tr_off + (16 * ks) * G::kPitch + mt * 64;
+        s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base));
+        s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base + 8 * G::kPitch));
+        u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
+        oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
+      }
+    }
+
+    if (t + 1 < n_tiles) store_stage(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- partial results: registers go out in their native order (coalesced), stats per head
+  float l_tot = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
+  const int64_t part = ((int64_t)(b * a.n_hblk + hb) * a.n_splits + sp);
+  float* wo = a.ws_o + (part * 4 + wave) * (int64_t)(8 * 16 * 64);
+#pragma unroll
+  for (int mt = 0; mt < 8; mt++)
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+      *reinterpret_cast<f32x4_t*>(wo + ((mt * 4 + c) * 64 + lane) * 4) =
+          f32x4_t{oacc[mt][4 * c], oacc[mt][4 * c + 1], oacc[mt][4 * c + 2], oacc[mt][4 * c + 3]};
+  if (dh == 0 && g == 0) {
+    float* ml = a.ws_ml + (part * 64 + hg * 32 + n) * 2;
+    ml[0] = m_run;
+    ml[1] = l_tot;
+  }
+}
+
+// Merge of the per-split partials: one workgroup per (batch, head block, wave slot, 32-column tile).
+template <int ODT>
+__global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int c = tid >> 6;  // accumulator quad: registers 4c..4c+3
+  const int mt = blockIdx.x & 7;
+  const int wave = (blockIdx.x >> 3) & 3;
+  const int bh = blockIdx.x >> 5;
+  const int hb = bh % a.n_hblk;
+  const int b = bh / a.n_hblk;
+  const int hg = wave >> 1, dh = wave & 1;
+  const int n = lane & 31, g = lane >> 5;
+  const int head = hb * 64 + hg * 32 + n;
+  if (head >= a.n_heads) return;
+
+  const float kLog2e = 1.4426950408889634f;
+  float sink = -__builtin_inff();
+  if (a.sinks) {
+    sink = (a.sinks_dtype == MSPR_F16 ? f16_bits_to_f32(reinterpret_cast<const uint16_t*>(a.sinks)[head])
+                                      : reinterpret_cast<const float*>(a.sinks)[head]) * kLog2e;
+  }
+  const int64_t part0 = (int64_t)(b * a.n_hblk + hb) * a.n_splits;
+  float m_all = sink;
+  for (int s = 0; s < a.n_splits; s++) m_all = fmaxf(m_all, a.ws_ml[((part0 + s) * 64 + hg * 32 + n) * 2]);
+  const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
+  float l = exp2f(sink - m_safe);
+  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < a.n_splits; s++) {
+    const float* ml = a.ws_ml + ((part0 + s) * 64 + hg * 32 + n) * 2;
+    float w = exp2f(ml[0] - m_safe);
+    l += ml[1] * w;
+    const float* wo = a.ws_o + ((part0 + s) * 4 + wave) * (int64_t)(8 * 16 * 64);
+    f32x4_t v = *reinterpret_cast<const f32x4_t*>(wo + ((mt * 4 + c) * 64 + lane) * 4);
+    o += v * w;
+  }
+  const float inv = l == 0.0f ? 0.0f : 1.0f / l;
+  float r[4] = {o.x * inv, o.y * inv, o.z * inv, o.w * inv};
+  const int dim0 = dh * 256 + 32 * mt + 8 * c + 4 * g;
+  const int64_t ooff = ((int64_t)b * a.n_heads + head) * kDV + dim0;
+  if constexpr (ODT == MSPR_F32) {
+    *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.out) + ooff) = f32x4_t{r[0], r[1], r[2], r[3]};
+  } else if constexpr (ODT == MSPR_BF16) {
+    u32x2_t w2 = {(uint32_t)f32_to_bf16_bits(r[0]) | ((uint32_t)f32_to_bf16_bits(r[1]) << 16),
+                  (uint32_t)f32_to_bf16_bits(r[2]) | ((uint32_t)f32_to_bf16_bits(r[3]) << 16)};
+    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + ooff) = w2;
+  } else {
+    float h[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) h[j] = f16_bits_to_f32(f32_to_f16_bits(r[j]));
+    if (a.rope && dim0 >= kDV - 64) {
+      // inverse partial rope on the float16 output at float16 op rounding
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        int p = (dim0 - (kDV - 64)) / 2 + j;
+        float theta = (float)a.params[0] * a.inv_freq[p];
+        float cs = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
+        float sn = f16_bits_to_f32(f32_to_f16_bits(-(float)sin((double)theta)));
+        float x0 = h[2 * j], x1 = h[2 * j + 1];
+        float m0 = f16_bits_to_f32(f32_to_f16_bits(x0 * cs)), m1 = f16_bits_to_f32(f32_to_f16_bits(x1 * sn));
+        float m2 = f16_bits_to_f32(f32_to_f16_bits(x0 * sn)), m3 = f16_bits_to_f32(f32_to_f16_bits(x1 * cs));
+        h[2 * j] = f16_bits_to_f32(f32_to_f16_bits(m0 - m1));
+        h[2 * j + 1] = f16_bits_to_f32(f32_to_f16_bits(m2 + m3));
+      }
+    }
+    u32x2_t w2 = {(uint32_t)f32_to_f16_bits(h[0]) | ((uint32_t)f32_to_f16_bits(h[1]) << 16),
+                  (uint32_t)f32_to_f16_bits(h[2]) | ((uint32_t)f32_to_f16_bits(h[3]) << 16)};
+    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + ooff) = w2;
+  }
+}
+
+int choose_splits(int batch_hblk, int n_keys) {
+  // enough workgroups to cover the 256 CUs, at least one 32-slot tile each, at most 64 splits
+  int tiles = (n_keys + kTile - 1) / kTile;
+  if (tiles < 1) tiles = 1;
+  int want = (256 + batch_hblk - 1) / batch_hblk;
+  if (want > 32) want = 32;
+  if (want > tiles) want = tiles;
+  if (want < 1) want = 1;
+  return want;
+}
+
+size_t workspace_bytes(int batch, int n_heads, int64_t n_keys) {
+  int n_hblk = (n_heads + 63) / 64;
+  int splits = choose_splits(batch * n_hblk, (int)n_keys);
+  size_t parts = (size_t)batch * n_hblk * splits;
+  return parts * (4 * 8 * 16 * 64 * sizeof(float)) + parts * 64 * 2 * sizeof(float) + 256;
+}
+
+template <int KDT, int DK>
+int launch_split(const SparseAttnArgs& a, hipStream_t st) {
+  using G = Geometry<DK>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_attn_split_kernel<KDT, DK>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes);
+    if (e != hipSuccess) {
+      mspr_set_error("sparse attention: cannot reserve %d bytes of LDS: %s", G::kLdsBytes, hipGetErrorString(e));
+      return MSPR_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  dim3 grid((unsigned)(a.batch * a.n_hblk * a.n_splits)), block(kThreads);
+  sparse_attn_split_kernel<KDT, DK><<<grid, block, G::kLdsBytes, st>>>(a);
+  MSPR_CHECK_LAUNCH("sparse attention (split)");
+  return MSPR_OK;
+}
+
+int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* workspace, size_t workspace_bytes_given,
+                         hipStream_t st) {
+  const int n_keys = a.n_win + a.n_idx;
+  a.n_hblk = (a.n_heads + 63) / 64;
+  a.n_splits = choose_splits(a.batch * a.n_hblk, n_keys);
+  int sps = (n_keys + a.n_splits - 1) / a.n_splits;
+  sps = (sps + 7) / 8 * 8;
+  if (sps < 8) sps = 8;
+  a.slots_per_split = sps;
+  size_t need = workspace_bytes(a.batch, a.n_heads, n_keys);
+  MSPR_REQUIRE(workspace && workspace_bytes_given >= need, "sparse attention: workspace of %zu bytes needed, %zu given",
+               need, workspace_bytes_given);
+  MSPR_REQUIRE(mspr_aligned(workspace, 16), "sparse attention: workspace must be 16-byte aligned");
+  size_t parts = (size_t)a.batch * a.n_hblk * a.n_splits;
+  a.ws_o = reinterpret_cast<float*>(workspace);
+  a.ws_ml = a.ws_o + parts * (4 * 8 * 16 * 64);
+  int rc;
+  if (kv_dtype == MSPR_BF16 && k_dim == 576) rc = launch_split<MSPR_BF16, 576>(a, st);
+  else if (kv_dtype == MSPR_BF16 && k_dim == 512) rc = launch_split<MSPR_BF16, 512>(a, st);
+  else if (kv_dtype == MSPR_F16 && k_dim == 576) rc = launch_split<MSPR_F16, 576>(a, st);
+  else rc = launch_split<MSPR_F16, 512>(a, st);
+  if (rc != MSPR_OK) return rc;
+  dim3 grid((unsigned)(a.batch * a.n_hblk * 32)), block(256);
+  if (a.out_dtype == MSPR_F32) sparse_attn_merge_kernel<MSPR_F32><<<grid, block, 0, st>>>(a);
+  else if (a.out_dtype == MSPR_BF16) sparse_attn_merge_kernel<MSPR_BF16><<<grid, block, 0, st>>>(a);
+  else sparse_attn_merge_kernel<MSPR_F16><<<grid, block, 0, st>>>(a);
+  MSPR_CHECK_LAUNCH("sparse attention (merge)");
+  return MSPR_OK;
+}
+
+}  // namespace
+
+extern "C" size_t mspr_sparse_attention_workspace_bytes(int batch, int n_heads, int64_t n_keys) {
+  if (batch < 1 || n_heads < 1 || n_keys < 0) return 0;
+  return workspace_bytes(batch, n_heads, n_keys);
+}
+
+extern "C" int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, const void* raw_kv, int raw_cap,
+                                                   const void* comp_kv, int64_t n_comp, const int32_t* topk,
+                                                   int top_k, const float* sinks, int64_t pos0, int window,
+                                                   int ratio, int raw_start, float* out, void* workspace,
+                                                   size_t workspace_bytes_given, void* stream) {
+  MSPR_REQUIRE(q && raw_kv && comp_kv && sinks && out, "indexed_mixed_attention_decode: null pointer");
+  MSPR_REQUIRE(top_k == 0 || topk, "indexed_mixed_attention_decode: null topk");
+  MSPR_REQUIRE(n_heads >= 1, "indexed_mixed_attention_decode: q must carry at least one head");
+  MSPR_REQUIRE(raw_cap >= 1, "indexed_mixed_attention_decode: raw_kv must contain at least one row");
+  MSPR_REQUIRE(raw_start >= 0 && raw_start < raw_cap, "indexed_mixed_attention_decode: raw_start must be inside raw_kv");
+  MSPR_REQUIRE(n_comp >= 1 && top_k >= 0 && window >= 0 && ratio >= 0 && pos0 >= 0 && pos0 < ((int64_t)1 << 31),
+               "indexed_mixed_attention_decode: bad size argument");
+  MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(raw_kv, 16) && mspr_aligned(comp_kv, 16) && mspr_aligned(out, 16),
+               "indexed_mixed_attention_decode: pointers must be 16-byte aligned");
+  // Ring rows visited, in the unsigned 32-bit arithmetic of the reference kernel
+  // (indexed_attention_kernel.py:120-141): a ring deeper than pos0+1 wraps and visits nothing.
+  uint32_t qpos = (uint32_t)pos0, n_raw = (uint32_t)raw_cap;
+  uint32_t first_raw_pos = qpos + 1u - n_raw;
+  uint32_t raw_last_pos = first_raw_pos + n_raw - 1u;
+  uint32_t window_first = (window != 0 && qpos + 1u > (uint32_t)window) ? qpos + 1u - (uint32_t)window : 0u;
+  uint32_t first = first_raw_pos > window_first ? first_raw_pos : window_first;
+  uint32_t last = qpos < raw_last_pos ? qpos : raw_last_pos;
+  SparseAttnArgs a = {};
+  a.q = q;
+  a.q_dtype = MSPR_F32;
+  a.q_batch_stride = 0;
+  a.n_heads = n_heads;
+  a.batch = 1;
+  a.win = raw_kv;
+  a.n_win = first <= last ? (int)(last - first + 1u) : 0;
+  a.win_first = first <= last ? (int)(first - first_raw_pos) : 0;
+  a.raw_start = raw_start;
+  a.raw_cap = raw_cap;
+  a.subst_row = nullptr;
+  a.subst_slot = -1;
+  a.pool = comp_kv;
+  a.n_pool = n_comp;
+  a.idx = topk;
+  a.n_idx = top_k;
+  int64_t visible = ratio == 0 ? n_comp : (pos0 + 1) / ratio;
+  a.visible = visible < n_comp ? visible : n_comp;
+  a.check_stop = 1;
+  a.sinks = sinks;
+  a.sinks_dtype = MSPR_F32;
+  a.scale_log2 = (float)(1.4426950408889634 / sqrt(512.0));
+  a.rope = 0;
+  a.out = out;
+  a.out_dtype = MSPR_F32;
+  return run_sparse_attention(a, MSPR_F16, 512, workspace, workspace_bytes_given, (hipStream_t)stream);
+}
+
+extern "C" int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* window, int window_rows,
+                                      const void* row, const void* pooled, int64_t n_rows, const int32_t* sel,
+                                      int n_sel, const void* sinks, const float* inv_freq, const int32_t* params,
+                                      float scale, void* out, void* workspace,
+                                      size_t workspace_bytes_given, void* stream) {
+  MSPR_REQUIRE(q && window && row && pooled && sinks && inv_freq && params && out,
+               "fused_decode_sdpa: null pointer");
+  MSPR_REQUIRE(n_sel == 0 || sel, "fused_decode_sdpa: null sel");
+  MSPR_REQUIRE(n_heads >= 1, "fused_decode_sdpa: q must carry at least one head");
+  MSPR_REQUIRE(window_rows >= 0 && n_rows >= 1 && n_sel >= 0, "fused_decode_sdpa: bad size argument");
+  MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(window, 16) && mspr_aligned(row, 16) && mspr_aligned(pooled, 16) &&
+                   mspr_aligned(out, 8),
+               "fused_decode_sdpa: pointers must be 16-byte aligned");
+  SparseAttnArgs a = {};
+  a.q = q;
+  a.q_dtype = MSPR_F16;
+  a.n_heads = n_heads;
+  a.batch = 1;
+  a.win = window;
+  a.n_win = window_rows;
+  a.win_first = 0;
+  a.raw_start = 0;
+  a.raw_cap = window_rows > 0 ? window_rows : 1;
+  a.subst_row = row;
+  a.subst_slot = -1;
+  a.subst_from_params = 1;
+  a.pool = pooled;
+  a.n_pool = n_rows;
+  a.idx = sel;
+  a.n_idx = n_sel;
+  a.visible = n_rows;
+  a.check_stop = 0;
+  a.sinks = sinks;
+  a.sinks_dtype = MSPR_F16;
+  a.scale_log2 = (float)((double)scale * 1.4426950408889634);
+  a.inv_freq = inv_freq;
+  a.params = params;
+  a.rope = 1;
+  a.out = out;
+  a.out_dtype = MSPR_F16;
+  return run_sparse_attention(a, MSPR_F16, 512, workspace, workspace_bytes_given, (hipStream_t)stream);
+}
+
+extern "C" int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, const float* sinks,
+                                      int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
+                                      int n_rows, int64_t win_start, int win_rows, float scale, void* out,
+                                      void* workspace, size_t workspace_bytes_given, void* stream) {
+  MSPR_REQUIRE(q && kv && out, "sparse_mla_decode: null pointer");
+  MSPR_REQUIRE(n_rows == 0 || rows, "sparse_mla_decode: null rows");
+  MSPR_REQUIRE(dtype == MSPR_F16 || dtype == MSPR_BF16, "sparse_mla_decode: dtype must be f16 or bf16");
+  MSPR_REQUIRE(k_dim == 512 || k_dim == 576, "sparse_mla_decode: k_dim must be 512 or 576");
+  MSPR_REQUIRE(v_dim == 512, "sparse_mla_decode: v_dim must be 512");
+  MSPR_REQUIRE(batch >= 1 && n_heads >= 1 && n_heads <= 128, "sparse_mla_decode: batch >= 1 and 1 <= n_heads <= 128");
+  MSPR_REQUIRE(n_pool >= 1 && n_pool < ((int64_t)1 << 31) && n_rows >= 0 && win_rows >= 0,
+               "sparse_mla_decode: bad size argument");
+  MSPR_REQUIRE(win_rows == 0 || (win_start >= 0 && win_start + win_rows <= n_pool),
+               "sparse_mla_decode: window must lie inside the pool");
+  MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(kv, 16) && mspr_aligned(out, 16),
+               "sparse_mla_decode: pointers must be 16-byte aligned");
+  SparseAttnArgs a = {};
+  a.q = q;
+  a.q_dtype = dtype;
+  a.q_batch_stride = (int64_t)n_heads * k_dim;
+  a.n_heads = n_heads;
+  a.batch = batch;
+  a.win = reinterpret_cast<const uint16_t*>(kv) + (win_rows > 0 ? win_start : 0) * k_dim;
+  a.win_batch_stride = n_pool * k_dim;
+  a.n_win = win_rows;
+  a.win_first = 0;
+  a.raw_start = 0;
+  a.raw_cap = win_rows > 0 ? win_rows : 1;
+  a.subst_row = nullptr;
+  a.subst_slot = -1;
+  a.pool = kv;
+  a.pool_batch_stride = n_pool * k_dim;
+  a.n_pool = n_pool;
+  a.idx = rows;
+  a.idx_batch_stride = n_rows;
+  a.n_idx = n_rows;
+  a.visible = n_pool;
+  a.check_stop = 0;
+  a.sinks = sinks;
+  a.sinks_dtype = MSPR_F32;
+  a.scale_log2 = (float)((double)scale * 1.4426950408889634);
+  a.rope = 0;
+  a.out = out;
+  a.out_dtype = dtype;
+  return run_sparse_attention(a, dtype, k_dim, workspace, workspace_bytes_given, (hipStream_t)stream);
+}
