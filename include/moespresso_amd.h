@@ -132,14 +132,28 @@ int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* window, int w
  * Every head of batch b attends rows kv[b, rows[b, :]] of a shared latent cache; K is the whole
  * k_dim-wide row and V its first v_dim columns.
  * q: [batch,n_heads,k_dim] of dtype (f16|bf16); kv: [batch,n_pool,k_dim] same dtype;
- * rows: int32 [batch,n_rows] gathered ids (negative or >= n_pool = skipped); the contiguous
+ * rows: int32 [batch,n_rows] gathered ids, pool row = id*row_mul + row_add (negative ids and rows
+ * outside the pool are skipped; row_mul 1, row_add 0 for plain row ids); the contiguous
  * window kv[b, win_start : win_start+win_rows] is attended as well (win_rows may be 0);
  * sinks: f32 [n_heads] or NULL; out: [batch,n_heads,v_dim] same dtype.
  * k_dim in {512,576}, v_dim = 512, n_heads <= 128. */
 int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, const float* sinks,
                            int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
-                           int n_rows, int64_t win_start, int win_rows, float scale, void* out,
-                           void* workspace, size_t workspace_bytes, void* stream);
+                           int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
+                           float scale, void* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------ measurement */
+
+/* Per-kernel GPU timing for benchmarks. Bit k of kernel_mask brackets every later launch of kernel
+ * k with HIP events on the launch stream (0 switches it off; it must be off under stream capture).
+ * Kernel ids: 1 fp8 indexer scores, 2 top-k, 3 sparse attention split, 4 sparse attention merge,
+ * 5 float32 indexer scores, 6 Q8 decode split, 7 Q8 decode merge, 8 flash prefill.
+ * No counterpart in the reference (its probes time whole calls on the host). */
+int mspr_profile_enable(int kernel_mask);
+
+/* Waits for the recorded launches of kernel_id, writes their durations in milliseconds to the HOST
+ * array ms_out (at most max_n) and forgets them; returns how many were written. */
+int mspr_profile_collect(int kernel_id, float* ms_out, int max_n);
 
 #ifdef __cplusplus
 }

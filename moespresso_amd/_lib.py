@@ -45,8 +45,29 @@ SIGNATURES = {
                 c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_sparse_mla_decode": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int64, c_int,
-                c_int64, c_int, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
+                c_int, c_int, c_int64, c_int, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mspr_profile_enable": (c_int, [c_int]),
+    "mspr_profile_collect": (c_int, [c_int, c_void_p, c_int]),
 }
+
+# kernel ids of mspr_profile_enable / mspr_profile_collect
+KERNEL_IDS = {"indexer_fp8": 1, "topk": 2, "sparse_split": 3, "sparse_merge": 4, "scores_f32": 5,
+              "q8_decode": 6, "q8_merge": 7, "flash_prefill": 8}
+
+
+def profile_enable(*names: str) -> None:
+    """Bracket later launches of the named kernels with HIP events (no names = off)."""
+    mask = 0
+    for n in names:
+        mask |= 1 << KERNEL_IDS[n]
+    lib().mspr_profile_enable(mask)
+
+
+def profile_collect(name: str, max_n: int = 65536) -> list[float]:
+    """Durations (ms) of the recorded launches of one kernel; waits for them and clears them."""
+    buf = (ctypes.c_float * max_n)()
+    n = lib().mspr_profile_collect(KERNEL_IDS[name], ctypes.cast(buf, c_void_p), max_n)
+    return [float(buf[i]) for i in range(n)]
 
 
 def sparse_attention_workspace(batch: int, n_heads: int, n_keys: int, device) -> torch.Tensor:

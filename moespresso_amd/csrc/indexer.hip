@@ -7,12 +7,18 @@
 // per-row head sum stays inside a lane (plus one xor-32 shuffle) and pool rows stream from HBM
 // straight into the B operand registers, 256 contiguous bytes per lane.
 #include "common.h"
+#include "profile.h"
 
 // The kernels in this file reproduce float32 operation sequences bit for bit: a multiply followed
 // by an add must round twice, so fused multiply-add contraction is off for the whole file.
 #pragma clang fp contract(off)
 
 namespace {
+
+// Separately rounded float32 multiply and add. They are defined below the pragma on purpose: the
+// HIP header intrinsics of the same purpose are inlined with contraction still allowed.
+__device__ __forceinline__ float mul_rn(float a, float b) { return a * b; }
+__device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
 
 constexpr float kHadamardScale = 0.08838834764831845f;  // float32(128^-1/2)
 constexpr float kAmaxFloor = 7.052966104933725e-38f;      // 6 * 2^-126
@@ -184,11 +190,11 @@ __global__ __launch_bounds__(256) void scores_f32_kernel(const void* __restrict_
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-      sum += __fmul_rn(__fmul_rn(fmaxf(acc0[i], 0.0f), scale), wl[0][i]);
+      sum += mul_rn(mul_rn(fmaxf(acc0[i], 0.0f), scale), wl[0][i]);
     }
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-      sum += __fmul_rn(__fmul_rn(fmaxf(acc1[i], 0.0f), scale), wl[1][i]);
+      sum += mul_rn(mul_rn(fmaxf(acc1[i], 0.0f), scale), wl[1][i]);
     }
     sum += __shfl_xor(sum, 32, MSPR_WAVE);
     if (g == 0 && row < n_rows) scores[row] = sum;
@@ -208,15 +214,15 @@ __global__ __launch_bounds__(256) void score_tail_kernel(const float* __restrict
   int64_t valid = pv < 0 ? 0 : (pv < capacity ? pv : capacity);
   float partial = 0.0f;
   for (int h = lane32; h < n_heads; h += 32) {
-    float w = __fmul_rn(load_as_f32<WDT>(wraw, h), head_norm);
+    float w = mul_rn(load_as_f32<WDT>(wraw, h), head_norm);
     float t = s[(int64_t)h * capacity + c];
     t = isnan(t) ? t : (t > 0.0f ? t : 0.0f);
-    t = __fmul_rn(t, scale);
-    t = __fmul_rn(t, w);
-    partial = __fadd_rn(partial, t);
+    t = mul_rn(t, scale);
+    t = mul_rn(t, w);
+    partial = add_rn(partial, t);
   }
 #pragma unroll
-  for (int off = 16; off >= 1; off >>= 1) partial = __fadd_rn(partial, __shfl_xor(partial, off, MSPR_WAVE));
+  for (int off = 16; off >= 1; off >>= 1) partial = add_rn(partial, __shfl_xor(partial, off, MSPR_WAVE));
   if (lane32 == 0 && col < capacity) neg[col] = col < valid ? -partial : __builtin_inff();
 }
 
@@ -246,7 +252,7 @@ __device__ __forceinline__ float fp8_roundtrip(float x, float scale) {
   n = (isnan(n) || n < 448.0f) ? n : 448.0f;
   float qv = e4m3_nearest_lower_ties(fabsf(n));
   float sign = n < 0.0f ? -1.0f : (n > 0.0f ? 1.0f : 0.0f);
-  return __fmul_rn(__fmul_rn(sign, qv), scale);
+  return mul_rn(mul_rn(sign, qv), scale);
 }
 
 // amax over a 64-element block = 4 lanes x 16 values.
@@ -356,6 +362,7 @@ int mspr_launch_scores_f32(const void* q, int q_dtype, int n_heads, const float*
   int64_t blocks = (n_tiles + 3) / 4;
   if (blocks > 2048) blocks = 2048;
   dim3 grid((unsigned)blocks), block(256);
+  MsprProfScope prof(MSPR_K_SCORES_F32, st);
 #define MSPR_SCORES_LAUNCH(DT)                                                                          \
   do {                                                                                                  \
     if (stage_half)                                                                                     \

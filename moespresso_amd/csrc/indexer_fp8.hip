@@ -9,6 +9,7 @@
 // 64 contiguous bytes of its key row, a wave 4 KB of contiguous memory per 32-key tile, and the
 // next tile is in flight while the current one is multiplied.
 #include "common.h"
+#include "profile.h"
 
 namespace {
 
@@ -116,9 +117,12 @@ int mspr_launch_indexer_scores_fp8(const void* q, const void* keys, const float*
   if (per_batch > max_blocks) per_batch = max_blocks;
   if (per_batch < 1) per_batch = 1;
   dim3 grid((unsigned)(per_batch * batch)), block(256);
-  indexer_scores_fp8_kernel<<<grid, block, 0, st>>>(reinterpret_cast<const uint16_t*>(q),
-                                                     reinterpret_cast<const uint8_t*>(keys), key_scales, weights,
-                                                     n_heads, n_rows, (int)per_batch, scores);
+  {
+    MsprProfScope prof(MSPR_K_INDEXER_FP8, st);
+    indexer_scores_fp8_kernel<<<grid, block, 0, st>>>(reinterpret_cast<const uint16_t*>(q),
+                                                       reinterpret_cast<const uint8_t*>(keys), key_scales, weights,
+                                                       n_heads, n_rows, (int)per_batch, scores);
+  }
   MSPR_CHECK_LAUNCH("indexer_scores_fp8");
   return MSPR_OK;
 }

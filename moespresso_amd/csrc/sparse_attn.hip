@@ -17,6 +17,7 @@
 // column = l % 32, row = 8*(i/4) + 4*(l/32) + i%4. In S^T the column is the head and the row the
 // key, so softmax statistics are per lane; P^T registers feed the next MFMA's B operand unchanged.
 #include "common.h"
+#include "profile.h"
 
 namespace {
 
@@ -50,6 +51,8 @@ struct SparseAttnArgs {
   int n_idx;
   int64_t visible;  // ids >= visible end the walk
   int check_stop;
+  int row_mul;  // pool row = id * row_mul + row_add
+  int row_add;
   // softmax
   const void* sinks;
   int sinks_dtype;
@@ -212,8 +215,10 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     int i = slot - a.n_win;
     if (i >= stop_pos) return nullptr;
     int id = idx_b[i];
-    if (id < 0 || (int64_t)id >= a.n_pool) return nullptr;
-    return pool_b + (int64_t)id * DK;
+    if (id < 0) return nullptr;
+    int64_t r = (int64_t)id * a.row_mul + a.row_add;
+    if (r < 0 || r >= a.n_pool) return nullptr;
+    return pool_b + r * DK;
   };
   u32x4_t stage[G::kLoads];
   bool stage_valid = false;
@@ -487,7 +492,10 @@ int launch_split(const SparseAttnArgs& a, hipStream_t st) {
     attr_set = true;
   }
   dim3 grid((unsigned)(a.batch * a.n_hblk * a.n_splits)), block(kThreads);
-  sparse_attn_split_kernel<KDT, DK><<<grid, block, G::kLdsBytes, st>>>(a);
+  {
+    MsprProfScope prof(MSPR_K_SPARSE_SPLIT, st);
+    sparse_attn_split_kernel<KDT, DK><<<grid, block, G::kLdsBytes, st>>>(a);
+  }
   MSPR_CHECK_LAUNCH("sparse attention (split)");
   return MSPR_OK;
 }
@@ -515,9 +523,12 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   else rc = launch_split<MSPR_F16, 512>(a, st);
   if (rc != MSPR_OK) return rc;
   dim3 grid((unsigned)(a.batch * a.n_hblk * 32)), block(256);
-  if (a.out_dtype == MSPR_F32) sparse_attn_merge_kernel<MSPR_F32><<<grid, block, 0, st>>>(a);
-  else if (a.out_dtype == MSPR_BF16) sparse_attn_merge_kernel<MSPR_BF16><<<grid, block, 0, st>>>(a);
-  else sparse_attn_merge_kernel<MSPR_F16><<<grid, block, 0, st>>>(a);
+  {
+    MsprProfScope prof(MSPR_K_SPARSE_MERGE, st);
+    if (a.out_dtype == MSPR_F32) sparse_attn_merge_kernel<MSPR_F32><<<grid, block, 0, st>>>(a);
+    else if (a.out_dtype == MSPR_BF16) sparse_attn_merge_kernel<MSPR_BF16><<<grid, block, 0, st>>>(a);
+    else sparse_attn_merge_kernel<MSPR_F16><<<grid, block, 0, st>>>(a);
+  }
   MSPR_CHECK_LAUNCH("sparse attention (merge)");
   return MSPR_OK;
 }
@@ -571,6 +582,8 @@ extern "C" int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, 
   int64_t visible = ratio == 0 ? n_comp : (pos0 + 1) / ratio;
   a.visible = visible < n_comp ? visible : n_comp;
   a.check_stop = 1;
+  a.row_mul = 1;
+  a.row_add = 0;
   a.sinks = sinks;
   a.sinks_dtype = MSPR_F32;
   a.scale_log2 = (float)(1.4426950408889634 / sqrt(512.0));
@@ -612,6 +625,8 @@ extern "C" int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* wi
   a.n_idx = n_sel;
   a.visible = n_rows;
   a.check_stop = 0;
+  a.row_mul = 1;
+  a.row_add = 0;
   a.sinks = sinks;
   a.sinks_dtype = MSPR_F16;
   a.scale_log2 = (float)((double)scale * 1.4426950408889634);
@@ -625,8 +640,9 @@ extern "C" int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* wi
 
 extern "C" int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, const float* sinks,
                                       int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
-                                      int n_rows, int64_t win_start, int win_rows, float scale, void* out,
-                                      void* workspace, size_t workspace_bytes_given, void* stream) {
+                                      int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
+                                      float scale, void* out, void* workspace, size_t workspace_bytes_given,
+                                      void* stream) {
   MSPR_REQUIRE(q && kv && out, "sparse_mla_decode: null pointer");
   MSPR_REQUIRE(n_rows == 0 || rows, "sparse_mla_decode: null rows");
   MSPR_REQUIRE(dtype == MSPR_F16 || dtype == MSPR_BF16, "sparse_mla_decode: dtype must be f16 or bf16");
@@ -661,6 +677,8 @@ extern "C" int mspr_sparse_mla_decode(const void* q, const void* kv, const int32
   a.n_idx = n_rows;
   a.visible = n_pool;
   a.check_stop = 0;
+  a.row_mul = row_mul;
+  a.row_add = row_add;
   a.sinks = sinks;
   a.sinks_dtype = MSPR_F32;
   a.scale_log2 = (float)((double)scale * 1.4426950408889634);

@@ -7,6 +7,7 @@
 // once; longer rows re-read global memory each pass. Histograms are private per wave (16 x 256
 // counters in LDS), so an LDS atomic only ever contends inside one wave.
 #include "common.h"
+#include "profile.h"
 
 namespace {
 
@@ -234,6 +235,7 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __re
 int mspr_launch_topk(const float* scores, int64_t score_stride, int batch, int64_t n_rows, int topk, int32_t* sel,
                      hipStream_t st) {
   dim3 grid((unsigned)batch), block(kThreads);
+  MsprProfScope prof(MSPR_K_TOPK, st);
   if (n_rows <= 8 * 1024) topk_select_kernel<8><<<grid, block, 0, st>>>(scores, score_stride, n_rows, topk, sel);
   else if (n_rows <= 32 * 1024) topk_select_kernel<32><<<grid, block, 0, st>>>(scores, score_stride, n_rows, topk, sel);
   else topk_select_kernel<0><<<grid, block, 0, st>>>(scores, score_stride, n_rows, topk, sel);

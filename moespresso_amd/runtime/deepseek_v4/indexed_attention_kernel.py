@@ -84,7 +84,7 @@ def indexed_mixed_attention_decode(q, raw_kv, comp_kv, topk, sinks, *, pos0: int
 
 
 def sparse_mla_decode(q, kv, rows, *, scale: float, v_dim: int = 512, window_start: int | None = None,
-                      window_rows: int = 0, sinks=None, workspace=None):
+                      window_rows: int = 0, sinks=None, workspace=None, row_mul: int = 1, row_add: int = 0):
     """Batched sparse multi-head-latent decode attention (BASELINE config 5 shape).
 
     Every head of batch entry ``b`` attends ``kv[b, rows[b, i]]`` for each
@@ -96,7 +96,10 @@ def sparse_mla_decode(q, kv, rows, *, scale: float, v_dim: int = 512, window_sta
     Args:
         q: ``[batch, n_heads, k_dim]`` float16 or bfloat16, ``k_dim`` 512 or 576.
         kv: ``[batch, n_pool, k_dim]`` same dtype.
-        rows: int32 ``[batch, n_rows]``; negative or out-of-range ids are skipped.
+        rows: int32 ``[batch, n_rows]`` gathered ids; the pool row of an id is
+            ``id * row_mul + row_add`` (so compressed-entry ids of a ratio-4
+            indexer address a per-token cache with ``row_mul=4, row_add=3``).
+            Negative ids and rows outside the pool are skipped.
         scale: softmax scale.
         sinks: optional float32 ``[n_heads]`` sink logits.
         workspace: optional float32 scratch from a previous call of the same shape.
@@ -139,7 +142,7 @@ def sparse_mla_decode(q, kv, rows, *, scale: float, v_dim: int = 512, window_sta
     ws = workspace if workspace is not None else _lib.sparse_attention_workspace(batch, n_heads, n_rows + window_rows, dev)
     rc = _lib.lib().mspr_sparse_mla_decode(
         _lib.ptr(qc), _lib.ptr(kc), _lib.ptr(rc_), _lib.ptr(sinks), _lib.DTYPE_CODE[q.dtype], batch, n_heads,
-        k_dim, 512, n_pool, n_rows, win_start, window_rows, float(scale), _lib.ptr(out), _lib.ptr(ws),
+        k_dim, 512, n_pool, n_rows, int(row_mul), int(row_add), win_start, window_rows, float(scale), _lib.ptr(out), _lib.ptr(ws),
         ws.numel() * 4, _lib.stream_ptr())
     _lib.check(rc, "sparse_mla_decode")
     return out

@@ -142,8 +142,11 @@ def test_sparse_mla_decode_matches_oracle(cfg):
     # oracle on the gathered rows (ids remapped to 0..R+W-1, skipped ids stay negative)
     local = np.where(all_rows >= 0, np.arange(all_rows.shape[1])[None, :], -1)
     want = ds4.sparse_mla_decode(q.float().cpu().numpy(), gathered, local, scale=scale)
-    err = np.abs(got.float().cpu().numpy() - want).max()
-    assert err < 2e-3, err
+    # 2e-3 absolute plus the half-precision rounding of the output itself (short row lists give
+    # outputs of magnitude ~1, where one bf16 ulp is 4e-3)
+    ulp = 2.0 ** -8 if cfg["dtype"] == "bf16" else 2.0 ** -11
+    err = np.abs(got.float().cpu().numpy() - want)
+    assert np.all(err <= 2e-3 + ulp * np.abs(want)), err.max()
 
 
 def test_sparse_mla_decode_full_config_batch16_with_sinks():
@@ -153,10 +156,11 @@ def test_sparse_mla_decode_full_config_batch16_with_sinks():
     kv = torch.randn((B, N, DK), device=dev(), generator=gen, dtype=torch.float32).to(torch.bfloat16)
     q = torch.randn((B, H, DK), device=dev(), generator=gen).to(torch.bfloat16)
     rng = np.random.default_rng(0)
-    rows = np.stack([4 * np.sort(rng.choice(32768 - 32, R, replace=False)) + 3 for _ in range(B)]).astype(np.int32)
+    ids = np.stack([np.sort(rng.choice(32768 - 32, R, replace=False)) for _ in range(B)]).astype(np.int32)
+    rows = 4 * ids + 3          # compressed-entry ids address the last token of their block
     sinks = rng.standard_normal(H).astype(np.float32)
-    got = iak.sparse_mla_decode(q, kv, to_dev(rows), scale=DK ** -0.5, window_start=N - W, window_rows=W,
-                                sinks=to_dev(sinks))
+    got = iak.sparse_mla_decode(q, kv, to_dev(ids), scale=DK ** -0.5, window_start=N - W, window_rows=W,
+                                sinks=to_dev(sinks), row_mul=4, row_add=3)
     all_rows = np.concatenate([np.tile(np.arange(N - W, N, dtype=np.int32), (B, 1)), rows], axis=1)
     gathered = np.stack([kv[b][torch.from_numpy(all_rows[b]).to(dev()).long()].float().cpu().numpy() for b in range(B)])
     local = np.tile(np.arange(all_rows.shape[1]), (B, 1))
