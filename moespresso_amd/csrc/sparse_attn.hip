@@ -83,14 +83,22 @@ __device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
   }
 }
 
+// Two float32 values rounded (nearest even) to the KV element type, packed in one register; the
+// vector conversion lowers to one v_cvt_pk_{bf16,f16}_f32.
 template <int KDT>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
   if constexpr (KDT == MSPR_BF16) {
-    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf2_t;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, bf2_t));
   } else {
-    return (uint32_t)f32_to_f16_bits(a) | ((uint32_t)f32_to_f16_bits(b) << 16);
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2_t;
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, h2_t));
   }
 }
+
+// 2^x through the hardware transcendental (no denormal fix-up: results below 2^-126 flush to 0,
+// which is what a softmax weight that small should do).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <int KDT>
 __device__ __forceinline__ float unpack_lo(uint32_t w) {
@@ -109,28 +117,9 @@ __device__ __forceinline__ float round_to_kdt(float v) {
   else return f16_bits_to_f32(f32_to_f16_bits(v));
 }
 
-// Eight consecutive query elements as one packed operand register group, converted to the KV type.
-template <int KDT>
-__device__ __forceinline__ void load_q8(const void* q, int q_dtype, int64_t off, float (&v)[8]) {
-  if (q_dtype == MSPR_F32) {
-    const f32x4_t* p = reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(q) + off);
-    f32x4_t a = p[0], b = p[1];
-    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
-    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-  } else {
-    u32x4_t w = *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(q) + off);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      if (q_dtype == MSPR_F16) {
-        v[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xFFFFu));
-        v[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
-      } else {
-        v[2 * j] = bf16_bits_to_f32((uint16_t)(w[j] & 0xFFFFu));
-        v[2 * j + 1] = bf16_bits_to_f32((uint16_t)(w[j] >> 16));
-      }
-    }
-  }
-}
+// Query element type of a kernel instance: the KV type itself (operands are used as loaded) or
+// float32 (rounded to the KV type on load).
+constexpr int kQSame = -1;
 
 template <int DK>
 struct Geometry {
@@ -144,7 +133,7 @@ struct Geometry {
   static constexpr int kLdsBytes = 2 * kTileBytes + 2 * kSxBytes + 2 * 32 * 4 + 2 * 4 + 16;
 };
 
-template <int KDT, int DK>
+template <int KDT, int DK, int QDT, bool ROPE>
 __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAttnArgs a) {
   using G = Geometry<DK>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -184,7 +173,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 
   // ---- prologue: stop position of the gathered walk, rope table
   if (tid == 0) *stop_shared = a.n_idx;
-  if (a.rope && tid < 32) {
+  if (ROPE && tid < 32) {
     float theta = (float)a.params[0] * a.inv_freq[tid];
     rope_c[tid] = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
     rope_s[tid] = f16_bits_to_f32(f32_to_f16_bits((float)sin((double)theta)));
@@ -205,16 +194,20 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   // ---- loader role: thread owns row r of the tile and chunks sub, sub+8, ...
   const int lrow = tid >> 3;
   const int lsub = tid & 7;
-  auto slot_src = [&](int slot) -> const uint16_t* {
+  // Row ids of the gathered segment are fetched one tile ahead of the rows themselves, so the
+  // dependent load (id -> row address) never sits in front of the MFMA work of a tile.
+  auto slot_id = [&](int slot) -> int {
+    int i = slot - a.n_win;
+    if (slot >= slot1 || i < 0 || i >= stop_pos) return -1;
+    return idx_b[i];
+  };
+  auto slot_src = [&](int slot, int id) -> const uint16_t* {
     if (slot >= slot1) return nullptr;
     if (slot < a.n_win) {
       if (slot == subst_slot) return reinterpret_cast<const uint16_t*>(a.subst_row);
-      int r = (int)(((int64_t)a.raw_start + a.win_first + slot) % a.raw_cap);
+      int r = (int)(((uint32_t)a.raw_start + (uint32_t)a.win_first + (uint32_t)slot) % (uint32_t)a.raw_cap);
       return win_b + (int64_t)r * DK;
     }
-    int i = slot - a.n_win;
-    if (i >= stop_pos) return nullptr;
-    int id = idx_b[i];
     if (id < 0) return nullptr;
     int64_t r = (int64_t)id * a.row_mul + a.row_add;
     if (r < 0 || r >= a.n_pool) return nullptr;
@@ -222,8 +215,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   };
   u32x4_t stage[G::kLoads];
   bool stage_valid = false;
-  auto issue_loads = [&](int tile) {
-    const uint16_t* src = slot_src(slot0 + tile * kTile + lrow);
+  auto issue_loads = [&](int tile, int id) {
+    const uint16_t* src = slot_src(slot0 + tile * kTile + lrow, id);
     stage_valid = src != nullptr;
     if (stage_valid) {
       const u32x4_t* p = reinterpret_cast<const u32x4_t*>(src);
@@ -248,41 +241,83 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     }
   };
 
-  if (n_tiles > 0) issue_loads(0);
+  int id_next = -1;
+  if (n_tiles > 0) {
+    issue_loads(0, slot_id(slot0 + lrow));
+    id_next = slot_id(slot0 + kTile + lrow);
+  }
 
   // ---- query operand: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7] per k-step
   const int head = hb * 64 + hg * 32 + n;
   u32x4_t qf[G::kSteps];
   {
     const bool live = head < a.n_heads;
-    const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)(live ? head : 0) * DK;
+    const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)(live ? head : 0) * DK + dh * G::kHalf + 8 * g;
+    if constexpr (QDT == kQSame && !ROPE) {
+      // operands are used as stored: all loads go out back to back
+      const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
 #pragma unroll
-    for (int ks = 0; ks < G::kSteps; ks++) {
-      const int d0 = dh * G::kHalf + 16 * ks + 8 * g;
-      float v[8];
-      load_q8<KDT>(a.q, a.q_dtype, qoff + d0, v);
+      for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = *reinterpret_cast<const u32x4_t*>(qp + 16 * ks);
+      if (!live) {
 #pragma unroll
-      for (int j = 0; j < 8; j++) v[j] = live ? round_to_kdt<KDT>(v[j]) : 0.0f;
-      if (a.rope && d0 >= DK - 64) {
-        // partial rope on interleaved pairs with every product and sum rounded to the element type
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          int p = (d0 - (DK - 64)) / 2 + j;
-          float c = rope_c[p], s = rope_s[p];
-          float x0 = v[2 * j], x1 = v[2 * j + 1];
-          float m0 = round_to_kdt<KDT>(x0 * c), m1 = round_to_kdt<KDT>(x1 * s);
-          float m2 = round_to_kdt<KDT>(x0 * s), m3 = round_to_kdt<KDT>(x1 * c);
-          v[2 * j] = round_to_kdt<KDT>(m0 - m1);
-          v[2 * j + 1] = round_to_kdt<KDT>(m2 + m3);
-        }
+        for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
       }
-      qf[ks] = u32x4_t{pack2<KDT>(v[0], v[1]), pack2<KDT>(v[2], v[3]), pack2<KDT>(v[4], v[5]), pack2<KDT>(v[6], v[7])};
+    } else {
+      float v[G::kSteps][8];
+      if constexpr (QDT == MSPR_F32) {
+        const float* qp = reinterpret_cast<const float*>(a.q) + qoff;
+        f32x4_t raw[G::kSteps][2];
+#pragma unroll
+        for (int ks = 0; ks < G::kSteps; ks++) {
+          raw[ks][0] = *reinterpret_cast<const f32x4_t*>(qp + 16 * ks);
+          raw[ks][1] = *reinterpret_cast<const f32x4_t*>(qp + 16 * ks + 4);
+        }
+#pragma unroll
+        for (int ks = 0; ks < G::kSteps; ks++)
+#pragma unroll
+          for (int j = 0; j < 8; j++) v[ks][j] = round_to_kdt<KDT>(raw[ks][j >> 2][j & 3]);
+      } else {
+        const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
+        u32x4_t raw[G::kSteps];
+#pragma unroll
+        for (int ks = 0; ks < G::kSteps; ks++) raw[ks] = *reinterpret_cast<const u32x4_t*>(qp + 16 * ks);
+#pragma unroll
+        for (int ks = 0; ks < G::kSteps; ks++)
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            v[ks][2 * j] = unpack_lo<KDT>(raw[ks][j]);
+            v[ks][2 * j + 1] = unpack_hi<KDT>(raw[ks][j]);
+          }
+      }
+#pragma unroll
+      for (int ks = 0; ks < G::kSteps; ks++) {
+        const int d0 = dh * G::kHalf + 16 * ks + 8 * g;
+        if (ROPE && d0 >= DK - 64) {
+          // partial rope on interleaved pairs with every product and sum rounded to the element type
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            int p = (d0 - (DK - 64)) / 2 + j;
+            float c = rope_c[p], s = rope_s[p];
+            float x0 = v[ks][2 * j], x1 = v[ks][2 * j + 1];
+            float m0 = round_to_kdt<KDT>(x0 * c), m1 = round_to_kdt<KDT>(x1 * s);
+            float m2 = round_to_kdt<KDT>(x0 * s), m3 = round_to_kdt<KDT>(x1 * c);
+            v[ks][2 * j] = round_to_kdt<KDT>(m0 - m1);
+            v[ks][2 * j + 1] = round_to_kdt<KDT>(m2 + m3);
+          }
+        }
+        qf[ks] = live ? u32x4_t{pack2<KDT>(v[ks][0], v[ks][1]), pack2<KDT>(v[ks][2], v[ks][3]),
+                                pack2<KDT>(v[ks][4], v[ks][5]), pack2<KDT>(v[ks][6], v[ks][7])}
+                      : u32x4_t{0u, 0u, 0u, 0u};
+      }
     }
   }
 
   f32x16_t oacc[8];
 #pragma unroll
   for (int mt = 0; mt < 8; mt++) oacc[mt] = f32x16_t{0};
+  // m_run is a lazily updated reference maximum: it only moves when a tile's maximum exceeds it by
+  // more than 8 (log2 units), so the 128 accumulator registers are rescaled a few times per kernel
+  // instead of once per tile; probabilities stay below 2^8.
   float m_run = -__builtin_inff();
   float l_run = 0.0f;
 
@@ -296,15 +331,26 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 
   for (int t = 0; t < n_tiles; t++) {
     const int buf = t & 1;
-    if (t + 1 < n_tiles) issue_loads(t + 1);
+    if (t + 1 < n_tiles) {
+      issue_loads(t + 1, id_next);
+      id_next = slot_id(slot0 + (t + 2) * kTile + lrow);
+    }
     const unsigned char* kt = kbuf + buf * G::kTileBytes;
 
     // S^T partial over this wave's half of the row width
     f32x16_t sacc = {0};
+    {
+      constexpr int kAhead = 6;  // LDS reads in flight in front of the dependent MFMA chain
+      u32x4_t af[kAhead];
 #pragma unroll
-    for (int ks = 0; ks < G::kSteps; ks++) {
-      u32x4_t af = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + ks * 32);
-      sacc = mfma32<KDT>(af, qf[ks], sacc);
+      for (int ks = 0; ks < kAhead; ks++) af[ks] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + ks * 32);
+#pragma unroll
+      for (int ks = 0; ks < G::kSteps; ks++) {
+        u32x4_t cur = af[ks % kAhead];
+        if (ks + kAhead < G::kSteps)
+          af[ks % kAhead] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + (ks + kAhead) * 32);
+        sacc = mfma32<KDT>(cur, qf[ks], sacc);
+      }
     }
     float* sxw = sx + (buf * 4 + wave) * (16 * 64);
 #pragma unroll
@@ -323,37 +369,51 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     }
 
     // online softmax in the log2 domain; key of register i is 8*(i/4) + 4g + i%4
-    const uint32_t mask = *reinterpret_cast<const uint32_t*>(vmask + buf * 4) >> (4 * g);
+    const uint32_t mask_all = *reinterpret_cast<const uint32_t*>(vmask + buf * 4);
     float tmax = -__builtin_inff();
+    if (mask_all == 0xFFFFFFFFu) {
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const bool valid = (mask >> (8 * (i / 4) + (i % 4))) & 1u;
-      float s = valid ? sacc[i] * a.scale_log2 : -__builtin_inff();
-      sacc[i] = s;
-      tmax = fmaxf(tmax, s);
+      for (int i = 0; i < 16; i++) {
+        sacc[i] *= a.scale_log2;
+        tmax = fmaxf(tmax, sacc[i]);
+      }
+    } else {
+      const uint32_t mask = mask_all >> (4 * g);
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const bool valid = (mask >> (8 * (i / 4) + (i % 4))) & 1u;
+        sacc[i] = valid ? sacc[i] * a.scale_log2 : -__builtin_inff();
+        tmax = fmaxf(tmax, sacc[i]);
+      }
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, MSPR_WAVE));
-    const float m_new = fmaxf(m_run, tmax);
-    const float m_safe = m_new == -__builtin_inff() ? 0.0f : m_new;
-    const float alpha = exp2f(m_run - m_safe);
+    // bf16 weights keep float32's exponent range, float16 weights must stay below 2^15
+    constexpr float kGrow = KDT == MSPR_BF16 ? 64.0f : 8.0f;
+    const bool grow = tmax > m_run + kGrow;
+    if (__any(grow)) {
+      const bool fresh = __all(m_run == -__builtin_inff());  // nothing accumulated yet
+      const float m_new = grow ? tmax : m_run;
+      const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
+      l_run *= alpha;
+      m_run = m_new;
+      if (!fresh) {
+#pragma unroll
+        for (int mt = 0; mt < 8; mt++) oacc[mt] = oacc[mt] * alpha;
+      }
+    }
+    const float m_safe = m_run == -__builtin_inff() ? 0.0f : m_run;
     float psum = 0.0f;
-    float p[16];
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-      p[i] = exp2f(sacc[i] - m_safe);
-      psum += p[i];
+      sacc[i] = fast_exp2(sacc[i] - m_safe);
+      psum += sacc[i];
     }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    if (!__all(alpha == 1.0f)) {
-#pragma unroll
-      for (int mt = 0; mt < 8; mt++) oacc[mt] = oacc[mt] * alpha;
-    }
+    l_run += psum;
     u32x4_t pf[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ks++)
-      pf[ks] = u32x4_t{pack2<KDT>(p[8 * ks], p[8 * ks + 1]), pack2<KDT>(p[8 * ks + 2], p[8 * ks + 3]),
-                       pack2<KDT>(p[8 * ks + 4], p[8 * ks + 5]), pack2<KDT>(p[8 * ks + 6], p[8 * ks + 7])};
+      pf[ks] = u32x4_t{pack2<KDT>(sacc[8 * ks], sacc[8 * ks + 1]), pack2<KDT>(sacc[8 * ks + 2], sacc[8 * ks + 3]),
+                       pack2<KDT>(sacc[8 * ks + 4], sacc[8 * ks + 5]), pack2<KDT>(sacc[8 * ks + 6], sacc[8 * ks + 7])};
 
     // O^T += V^T . P^T ; V^T operands through the LDS transpose read of the row-major tile
 #pragma unroll
@@ -412,18 +472,37 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
                                       : reinterpret_cast<const float*>(a.sinks)[head]) * kLog2e;
   }
   const int64_t part0 = (int64_t)(b * a.n_hblk + hb) * a.n_splits;
+  const float* ml0 = a.ws_ml + (part0 * 64 + hg * 32 + n) * 2;
+  const float* wo0 = a.ws_o + (part0 * 4 + wave) * (int64_t)(8 * 16 * 64) + ((mt * 4 + c) * 64 + lane) * 4;
+  constexpr int kChunk = 8;
   float m_all = sink;
-  for (int s = 0; s < a.n_splits; s++) m_all = fmaxf(m_all, a.ws_ml[((part0 + s) * 64 + hg * 32 + n) * 2]);
+  for (int s0 = 0; s0 < a.n_splits; s0 += kChunk) {
+    float mv[kChunk];
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) mv[j] = s0 + j < a.n_splits ? ml0[(int64_t)(s0 + j) * 128] : -__builtin_inff();
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) m_all = fmaxf(m_all, mv[j]);
+  }
   const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
   float l = exp2f(sink - m_safe);
   f32x4_t o = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < a.n_splits; s++) {
-    const float* ml = a.ws_ml + ((part0 + s) * 64 + hg * 32 + n) * 2;
-    float w = exp2f(ml[0] - m_safe);
-    l += ml[1] * w;
-    const float* wo = a.ws_o + ((part0 + s) * 4 + wave) * (int64_t)(8 * 16 * 64);
-    f32x4_t v = *reinterpret_cast<const f32x4_t*>(wo + ((mt * 4 + c) * 64 + lane) * 4);
-    o += v * w;
+  for (int s0 = 0; s0 < a.n_splits; s0 += kChunk) {
+    float mv[kChunk], lv[kChunk];
+    f32x4_t ov[kChunk];
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) {
+      const bool live = s0 + j < a.n_splits;
+      const int64_t sj = live ? s0 + j : 0;
+      mv[j] = live ? ml0[sj * 128] : -__builtin_inff();
+      lv[j] = ml0[sj * 128 + 1];
+      ov[j] = *reinterpret_cast<const f32x4_t*>(wo0 + sj * (int64_t)(4 * 8 * 16 * 64));
+    }
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) {
+      float w = exp2f(mv[j] - m_safe);
+      l += lv[j] * w;
+      o += ov[j] * w;
+    }
   }
   const float inv = l == 0.0f ? 0.0f : 1.0f / l;
   float r[4] = {o.x * inv, o.y * inv, o.z * inv, o.w * inv};
@@ -478,12 +557,12 @@ size_t workspace_bytes(int batch, int n_heads, int64_t n_keys) {
   return parts * (4 * 8 * 16 * 64 * sizeof(float)) + parts * 64 * 2 * sizeof(float) + 256;
 }
 
-template <int KDT, int DK>
+template <int KDT, int DK, int QDT, bool ROPE>
 int launch_split(const SparseAttnArgs& a, hipStream_t st) {
   using G = Geometry<DK>;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_attn_split_kernel<KDT, DK>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_attn_split_kernel<KDT, DK, QDT, ROPE>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes);
     if (e != hipSuccess) {
       mspr_set_error("sparse attention: cannot reserve %d bytes of LDS: %s", G::kLdsBytes, hipGetErrorString(e));
@@ -494,7 +573,7 @@ int launch_split(const SparseAttnArgs& a, hipStream_t st) {
   dim3 grid((unsigned)(a.batch * a.n_hblk * a.n_splits)), block(kThreads);
   {
     MsprProfScope prof(MSPR_K_SPARSE_SPLIT, st);
-    sparse_attn_split_kernel<KDT, DK><<<grid, block, G::kLdsBytes, st>>>(a);
+    sparse_attn_split_kernel<KDT, DK, QDT, ROPE><<<grid, block, G::kLdsBytes, st>>>(a);
   }
   MSPR_CHECK_LAUNCH("sparse attention (split)");
   return MSPR_OK;
@@ -517,10 +596,12 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   a.ws_o = reinterpret_cast<float*>(workspace);
   a.ws_ml = a.ws_o + parts * (4 * 8 * 16 * 64);
   int rc;
-  if (kv_dtype == MSPR_BF16 && k_dim == 576) rc = launch_split<MSPR_BF16, 576>(a, st);
-  else if (kv_dtype == MSPR_BF16 && k_dim == 512) rc = launch_split<MSPR_BF16, 512>(a, st);
-  else if (kv_dtype == MSPR_F16 && k_dim == 576) rc = launch_split<MSPR_F16, 576>(a, st);
-  else rc = launch_split<MSPR_F16, 512>(a, st);
+  if (a.rope) rc = launch_split<MSPR_F16, 512, kQSame, true>(a, st);
+  else if (a.q_dtype == MSPR_F32) rc = launch_split<MSPR_F16, 512, MSPR_F32, false>(a, st);
+  else if (kv_dtype == MSPR_BF16 && k_dim == 576) rc = launch_split<MSPR_BF16, 576, kQSame, false>(a, st);
+  else if (kv_dtype == MSPR_BF16 && k_dim == 512) rc = launch_split<MSPR_BF16, 512, kQSame, false>(a, st);
+  else if (kv_dtype == MSPR_F16 && k_dim == 576) rc = launch_split<MSPR_F16, 576, kQSame, false>(a, st);
+  else rc = launch_split<MSPR_F16, 512, kQSame, false>(a, st);
   if (rc != MSPR_OK) return rc;
   dim3 grid((unsigned)(a.batch * a.n_hblk * 32)), block(256);
   {

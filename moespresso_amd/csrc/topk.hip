@@ -1,11 +1,17 @@
-// Deterministic top-k over float32 score rows: four-pass MSB radix select on monotone uint32
-// keys, then ordered emission (rows strictly above the k-th key in ascending row order, then the
-// lowest-index rows tied with it).
+// Deterministic top-k over float32 score rows: MSB radix select on monotone uint32 keys (four
+// 8-bit digits), then ordered emission (rows strictly above the k-th key in ascending row order,
+// then the lowest-index rows tied with it).
 //
 // One 1024-thread workgroup per score row. For rows of up to CACHE*1024 scores every thread keeps
 // its keys in registers (striped ownership: thread t owns rows t, t+1024, ...), so HBM/L2 is read
-// once; longer rows re-read global memory each pass. Histograms are private per wave (16 x 256
-// counters in LDS), so an LDS atomic only ever contends inside one wave.
+// once; longer rows re-read global memory each pass.
+//
+// Histograms: 256 bins x 64 copies in LDS, copy = lane id, laid out [bin][copy]. Every lane of an
+// LDS atomic then hits its own bank whatever the digit distribution is (scores of one row usually
+// share their top byte, which would serialise a single shared counter 64-fold).
+//
+// After the first two digits the keys that still match the 16-bit prefix are usually a handful;
+// they are compacted into an LDS list and the last two digits run on that list only.
 #include "common.h"
 #include "profile.h"
 
@@ -13,17 +19,63 @@ namespace {
 
 constexpr int kThreads = 1024;
 constexpr int kWaves = kThreads / 64;
+constexpr int kCopies = 64;
+constexpr int kListCap = 2048;
 
 struct SelectState {
   uint32_t prefix;
   uint32_t need;
+  uint32_t live;   // keys matching the current prefix
+  uint32_t list_n;
 };
+
+// Wave 0: pick the bucket where the count from the top first reaches `need`. totals[b] in LDS.
+__device__ __forceinline__ void choose_bucket(const uint32_t* totals, SelectState* st, uint32_t shift, int lane) {
+  uint32_t t[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) t[j] = totals[4 * lane + j];
+  uint32_t lane_sum = t[0] + t[1] + t[2] + t[3];
+  uint32_t sfx = lane_sum;  // inclusive suffix sum over lanes
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    uint32_t o = __shfl_down(sfx, off, MSPR_WAVE);
+    if (lane + off < 64) sfx += o;
+  }
+  const uint32_t need = st->need;
+  const uint32_t prefix = st->prefix;
+  int chosen = -1;
+  uint32_t chosen_need = 0u, chosen_cnt = 0u;
+  uint32_t run = sfx - lane_sum;  // keys in buckets of higher lanes
+#pragma unroll
+  for (int j = 3; j >= 0; j--) {
+    if (chosen < 0 && run < need && run + t[j] >= need) {
+      chosen = 4 * lane + j;
+      chosen_need = need - run;
+      chosen_cnt = t[j];
+    }
+    run += t[j];
+  }
+  uint64_t any = __ballot(chosen >= 0);
+  if (any == 0ull) {
+    // fewer live keys than needed cannot happen for topk <= n_rows; bucket 0 takes the rest
+    if (lane == 0) {
+      st->need = need - (sfx - t[0]);
+      st->live = t[0];
+    }
+  } else if (chosen >= 0) {
+    st->prefix = prefix | ((uint32_t)chosen << shift);
+    st->need = chosen_need;
+    st->live = chosen_cnt;
+  }
+}
 
 template <int CACHE>
 __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __restrict__ scores_all,
                                                                 int64_t score_stride, int64_t n_rows, int topk,
                                                                 int32_t* __restrict__ sel_all) {
-  __shared__ uint32_t hist[kWaves * 256];
+  __shared__ uint32_t hist[256 * kCopies];  // [bin][copy]
+  __shared__ uint32_t totals[256];
+  __shared__ uint32_t list[kListCap];
   __shared__ SelectState st;
   __shared__ uint32_t cnt_above[kThreads];
   __shared__ uint32_t cnt_tie[kThreads];
@@ -37,10 +89,8 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __re
   int32_t* sel = sel_all + (int64_t)blockIdx.x * topk;
   const int64_t n_chunks = (n_rows + kThreads - 1) / kThreads;
 
-  // keys of padding slots never match a live prefix group and never pass the threshold tests:
-  // they are skipped through the `live` flag instead of a sentinel value.
   uint32_t kreg[CACHE > 0 ? CACHE : 1];
-  if (CACHE > 0) {
+  if constexpr (CACHE > 0) {
 #pragma unroll
     for (int i = 0; i < CACHE; i++) {
       int64_t r = (int64_t)i * kThreads + tid;
@@ -50,79 +100,91 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __re
   if (tid == 0) {
     st.prefix = 0u;
     st.need = (uint32_t)topk;
+    st.live = (uint32_t)n_rows;
+    st.list_n = 0u;
   }
 
-  for (int pass = 0; pass < 4; pass++) {
+  // one digit over every key: count keys whose higher digits equal the prefix
+  auto full_pass = [&](int pass) {
     const uint32_t shift = 24u - 8u * pass;
-    for (int i = tid; i < kWaves * 256; i += kThreads) hist[i] = 0u;
+    u32x4_t* h4 = reinterpret_cast<u32x4_t*>(hist);
+    for (int i = tid; i < 256 * kCopies / 4; i += kThreads) h4[i] = u32x4_t{0u, 0u, 0u, 0u};
     __syncthreads();
     const uint32_t prefix = st.prefix;
     const uint32_t mask_hi = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8u));
-    uint32_t* myhist = hist + wave * 256;
-    if (CACHE > 0) {
+    if constexpr (CACHE > 0) {
 #pragma unroll
       for (int i = 0; i < CACHE; i++) {
         int64_t r = (int64_t)i * kThreads + tid;
         uint32_t key = kreg[i];
-        if (r < n_rows && (key & mask_hi) == prefix) atomicAdd(&myhist[(key >> shift) & 0xFFu], 1u);
+        if (r < n_rows && (key & mask_hi) == prefix) atomicAdd(&hist[((key >> shift) & 0xFFu) * kCopies + lane], 1u);
       }
     } else {
       for (int64_t c = 0; c < n_chunks; c++) {
         int64_t r = c * kThreads + tid;
         if (r < n_rows) {
           uint32_t key = score_key(scores[r]);
-          if ((key & mask_hi) == prefix) atomicAdd(&myhist[(key >> shift) & 0xFFu], 1u);
+          if ((key & mask_hi) == prefix) atomicAdd(&hist[((key >> shift) & 0xFFu) * kCopies + lane], 1u);
         }
       }
     }
     __syncthreads();
-    if (wave == 0) {
-      // lane l owns buckets 4l..4l+3; suffix sums from bucket 255 downward
-      uint32_t t[4];
+    // totals[bin] = sum over copies: four threads per bin, 16 copies each, rotated to spread banks
+    {
+      const int bin = tid >> 2, q = tid & 3;
+      uint32_t s = 0u;
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        uint32_t s = 0u;
-        for (int w = 0; w < kWaves; w++) s += hist[w * 256 + 4 * lane + j];
-        t[j] = s;
+      for (int j = 0; j < 16; j++) s += hist[bin * kCopies + q * 16 + ((j + lane) & 15)];
+      s += __shfl_xor(s, 1, MSPR_WAVE);
+      s += __shfl_xor(s, 2, MSPR_WAVE);
+      if (q == 0) totals[bin] = s;
+    }
+    __syncthreads();
+    if (wave == 0) choose_bucket(totals, &st, shift, lane);
+    __syncthreads();
+  };
+
+  full_pass(0);
+  full_pass(1);
+
+  if (st.live <= (uint32_t)kListCap) {
+    // compact the keys that match the 16-bit prefix; their order does not matter here
+    const uint32_t prefix = st.prefix;
+    if constexpr (CACHE > 0) {
+#pragma unroll
+      for (int i = 0; i < CACHE; i++) {
+        int64_t r = (int64_t)i * kThreads + tid;
+        uint32_t key = kreg[i];
+        if (r < n_rows && (key & 0xFFFF0000u) == prefix) list[atomicAdd(&st.list_n, 1u)] = key;
       }
-      uint32_t lane_sum = t[0] + t[1] + t[2] + t[3];
-      // inclusive suffix scan over lanes: sfx = sum of lane_sum over lanes >= lane
-      uint32_t sfx = lane_sum;
-#pragma unroll
-      for (int off = 1; off < 64; off <<= 1) {
-        uint32_t o = __shfl_down(sfx, off, MSPR_WAVE);
-        if (lane + off < 64) sfx += o;
-      }
-      const uint32_t need = st.need;
-      uint32_t above_lane = sfx - lane_sum;  // count in buckets of higher lanes
-      // walk this lane's buckets from the top: bucket b is chosen when the count at or above b
-      // first reaches `need`
-      int chosen = -1;
-      uint32_t chosen_need = 0u;
-      uint32_t run = above_lane;
-#pragma unroll
-      for (int j = 3; j >= 0; j--) {
-        if (chosen < 0 && run < need && run + t[j] >= need) {
-          chosen = 4 * lane + j;
-          chosen_need = need - run;
+    } else {
+      for (int64_t c = 0; c < n_chunks; c++) {
+        int64_t r = c * kThreads + tid;
+        if (r < n_rows) {
+          uint32_t key = score_key(scores[r]);
+          if ((key & 0xFFFF0000u) == prefix) list[atomicAdd(&st.list_n, 1u)] = key;
         }
-        run += t[j];
-      }
-      // exactly one lane chooses when the live count >= need; otherwise bucket 0 takes the rest
-      uint64_t any = __ballot(chosen >= 0);
-      if (any == 0ull) {
-        if (lane == 0) {
-          // count above bucket 0 = total - t[0]
-          uint32_t total = sfx;
-          st.prefix = prefix;  // bucket 0 adds no bits
-          st.need = need - (total - t[0]);
-        }
-      } else if (chosen >= 0) {
-        st.prefix = prefix | ((uint32_t)chosen << shift);
-        st.need = chosen_need;
       }
     }
     __syncthreads();
+    const uint32_t n_list = st.list_n;
+    for (int pass = 2; pass < 4; pass++) {
+      const uint32_t shift = 24u - 8u * pass;
+      if (tid < 256) totals[tid] = 0u;
+      __syncthreads();
+      const uint32_t pfx = st.prefix;
+      const uint32_t mask_hi = 0xFFFFFFFFu << (shift + 8u);
+      for (uint32_t i = tid; i < n_list; i += kThreads) {
+        uint32_t key = list[i];
+        if ((key & mask_hi) == pfx) atomicAdd(&totals[(key >> shift) & 0xFFu], 1u);
+      }
+      __syncthreads();
+      if (wave == 0) choose_bucket(totals, &st, shift, lane);
+      __syncthreads();
+    }
+  } else {
+    full_pass(2);
+    full_pass(3);
   }
 
   const uint32_t threshold = st.prefix;
@@ -159,7 +221,6 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __re
   };
   for (int64_t g0 = 0; g0 < n_chunks; g0 += 64) {
     const int gchunks = (int)((n_chunks - g0) < 64 ? (n_chunks - g0) : 64);
-    // E1: ballots per chunk
     if constexpr (CACHE > 0) {
 #pragma unroll
       for (int ci = 0; ci < CACHE; ci++) {
@@ -180,7 +241,7 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __re
       cnt_tie[i] = 0u;
     }
     __syncthreads();
-    // E2: exclusive scan over the (chunk, wave) entries, one per thread
+    // exclusive scan over the (chunk, wave) entries, one per thread
     uint32_t va = cnt_above[tid], vt = cnt_tie[tid];
     uint32_t ia = va, it = vt;
 #pragma unroll
@@ -210,7 +271,6 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __re
       carry[1] = base_t + it;
     }
     __syncthreads();
-    // E3: emit
     if constexpr (CACHE > 0) {
 #pragma unroll
       for (int ci = 0; ci < CACHE; ci++) {
