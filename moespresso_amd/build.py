@@ -26,6 +26,8 @@ COMMON_FLAGS = [
     # packed FP32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # the asynchronous LDS loads set M0 by hand inside inline asm
+    "-Wno-inline-asm",
 ]
 
 

@@ -19,6 +19,20 @@
 #include "common.h"
 #include "profile.h"
 
+#ifdef MSPR_SPARSE_TRACE
+// Debug build only: per-workgroup cycle stamps of the split kernel's phases.
+static long long* g_trace_buf = nullptr;
+extern "C" void mspr_debug_set_trace(long long* p) { g_trace_buf = p; }
+#define MSPR_STAMP(i)                                                         \
+  do {                                                                        \
+    if (a.trace && tid == 0) a.trace[(int64_t)blockIdx.x * 64 + (i)] = clock64(); \
+  } while (0)
+#else
+#define MSPR_STAMP(i) \
+  do {                \
+  } while (0)
+#endif
+
 namespace {
 
 constexpr int kTile = 32;
@@ -70,6 +84,7 @@ struct SparseAttnArgs {
   // output
   void* out;
   int out_dtype;
+  long long* trace;  // debug builds only
 };
 
 template <int KDT>
@@ -121,28 +136,65 @@ __device__ __forceinline__ float round_to_kdt(float v) {
 // float32 (rounded to the KV type on load).
 constexpr int kQSame = -1;
 
+// A zero row for slots that are skipped: the asynchronous tile loads always run with every lane
+// active (the wait counters below rely on a fixed number of loads per tile), so a skipped slot reads
+// zeros instead of being predicated off.
+__device__ __attribute__((aligned(16))) const unsigned char g_zero_row[1280] = {0};
+
+#define MSPR_GLB_PTR(T, p) ((__attribute__((address_space(1))) T*)(p))
+
+// Wait until at most N of this wave's vector-memory operations are outstanding and all of its LDS
+// operations are done, then meet the other waves. Written as one asm statement so that no
+// compiler-inserted full drain (as a fence would add) sits between the asynchronous tile loads.
+template <int N>
+__device__ __forceinline__ void wait_vm_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+// One wave-wide asynchronous copy global -> LDS: lane i's 16 bytes at `src` land at lds_base + 16 i
+// (lds_base is wave-uniform). Issued through asm so that the compiler's wait-count pass does not
+// see LDS writes in flight (it would drain them in front of every LDS transpose read); completion
+// is awaited explicitly through wait_vm_and_barrier.
+__device__ __forceinline__ void async_load_16(uint64_t src, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <int DK>
 struct Geometry {
-  static constexpr int kChunks = DK / 8;          // 16-byte chunks per row
-  static constexpr int kLoads = kChunks / 8;      // per loader thread (8 threads per row)
-  static constexpr int kPitch = DK * 2 + 16;      // bytes; +16 keeps 8 consecutive rows on distinct 16B bank groups
-  static constexpr int kHalf = DK / 2;            // contraction columns per dh wave
-  static constexpr int kSteps = kHalf / 16;       // MFMA k-steps per dh wave
-  static constexpr int kTileBytes = kTile * kPitch;
-  static constexpr int kSxBytes = 4 * 16 * 64 * 4;  // 4 waves x 16 floats x 64 lanes
-  static constexpr int kLdsBytes = 2 * kTileBytes + 2 * kSxBytes + 2 * 32 * 4 + 2 * 4 + 16;
+  static constexpr int kSlots = DK / 8 + 1;        // 16-byte slots per LDS row; the last one is padding, so
+                                                   // 8 consecutive rows start on distinct 16B bank groups
+  static constexpr int kPitch = kSlots * 16;       // bytes
+  static constexpr int kTileSlots = kTile * kSlots;
+  static constexpr int kInstr = (kTileSlots + 63) / 64;   // wave-wide 1 KB loads per tile
+  static constexpr int kPerThread = (kInstr + 3) / 4;     // loads per thread per tile (wave 0 issues the odd one)
+  static constexpr int kTileBytes = kInstr * 1024;
+  static constexpr int kHalf = DK / 2;             // contraction columns per dh wave
+  static constexpr int kSteps = kHalf / 16;        // MFMA k-steps per dh wave
+  static constexpr int kBufs = 3;                  // tile ring: one in use, two in flight
+  static constexpr int kSxBytes = 4 * 16 * 64 * 4; // 4 waves x 16 floats x 64 lanes
+  static constexpr int kMaxIds = 1024;             // gathered slots per workgroup
+  static constexpr int kOffSx = kBufs * kTileBytes;
+  static constexpr int kOffRowPtr = kOffSx + 2 * kSxBytes;
+  static constexpr int kOffVmask = kOffRowPtr + kBufs * kTile * 8;
+  static constexpr int kOffIds = kOffVmask + 16;
+  static constexpr int kOffRope = kOffIds + kMaxIds * 4;
+  static constexpr int kOffStop = kOffRope + 64 * 4;
+  static constexpr int kLdsBytes = kOffStop + 16;
+  static_assert(kInstr % 4 == 1, "wave 0 issues exactly one load more than the other waves");
 };
 
 template <int KDT, int DK, int QDT, bool ROPE>
 __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAttnArgs a) {
   using G = Geometry<DK>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  unsigned char* kbuf = lds;                                       // [2][kTile][kPitch]
-  float* sx = reinterpret_cast<float*>(lds + 2 * G::kTileBytes);   // [2][4][16*64]
-  float* rope_c = reinterpret_cast<float*>(lds + 2 * G::kTileBytes + 2 * G::kSxBytes);
+  unsigned char* kbuf = lds;                                                   // [kBufs][kTileBytes]
+  float* sx = reinterpret_cast<float*>(lds + G::kOffSx);                       // [2][4][16*64]
+  uint64_t* rowptr = reinterpret_cast<uint64_t*>(lds + G::kOffRowPtr);         // [kBufs][kTile]
+  uint32_t* vmask = reinterpret_cast<uint32_t*>(lds + G::kOffVmask);           // [4]
+  int32_t* ids = reinterpret_cast<int32_t*>(lds + G::kOffIds);                 // [kMaxIds]
+  float* rope_c = reinterpret_cast<float*>(lds + G::kOffRope);
   float* rope_s = rope_c + 32;
-  uint8_t* vmask = reinterpret_cast<uint8_t*>(rope_s + 32);        // [2][4] one byte per wave per buffer
-  int* stop_shared = reinterpret_cast<int*>(vmask + 8);
+  int* stop_shared = reinterpret_cast<int*>(lds + G::kOffStop);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -171,15 +223,36 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   const uint16_t* pool_b = reinterpret_cast<const uint16_t*>(a.pool) + (int64_t)b * a.pool_batch_stride;
   const int32_t* idx_b = a.idx + (int64_t)b * a.idx_batch_stride;
 
-  // ---- prologue: stop position of the gathered walk, rope table
-  if (tid == 0) *stop_shared = a.n_idx;
+  MSPR_STAMP(0);
+  // ---- query operand loads go out first: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7]
+  const int head = hb * 64 + hg * 32 + n;
+  const bool q_live = head < a.n_heads;
+  const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)(q_live ? head : 0) * DK + dh * G::kHalf + 8 * g;
+  u32x4_t qf[G::kSteps];
+  f32x4_t qraw32[QDT == MSPR_F32 ? G::kSteps : 1][2];
+  if constexpr (QDT == MSPR_F32) {
+    const float* qp = reinterpret_cast<const float*>(a.q) + qoff;
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) {
+      qraw32[ks][0] = *reinterpret_cast<const f32x4_t*>(qp + 16 * ks);
+      qraw32[ks][1] = *reinterpret_cast<const f32x4_t*>(qp + 16 * ks + 4);
+    }
+  } else {
+    const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = *reinterpret_cast<const u32x4_t*>(qp + 16 * ks);
+  }
+
+  // ---- stop position of the gathered walk, rope table, gathered ids of this slot range
   if (ROPE && tid < 32) {
     float theta = (float)a.params[0] * a.inv_freq[tid];
     rope_c[tid] = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
     rope_s[tid] = f16_bits_to_f32(f32_to_f16_bits((float)sin((double)theta)));
   }
-  __syncthreads();
+  int stop_pos = a.n_idx;
   if (a.check_stop) {
+    if (tid == 0) *stop_shared = a.n_idx;
+    __syncthreads();
     int first = a.n_idx;
     for (int i = tid; i < a.n_idx; i += kThreads) {
       int id = idx_b[i];
@@ -187,156 +260,161 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     }
     if (first < a.n_idx) atomicMin(stop_shared, first);
     __syncthreads();
+    stop_pos = *stop_shared;
   }
-  const int stop_pos = *stop_shared;
   const int subst_slot = a.subst_from_params ? a.params[1] : a.subst_slot;
+  const int id_base = slot0 > a.n_win ? slot0 - a.n_win : 0;           // first gathered index of the range
+  const int id_count = slot1 > a.n_win ? slot1 - a.n_win - id_base : 0;  // <= kMaxIds by construction
+  for (int i = tid; i < id_count; i += kThreads) ids[i] = id_base + i < stop_pos ? idx_b[id_base + i] : -1;
 
-  // ---- loader role: thread owns row r of the tile and chunks sub, sub+8, ...
-  const int lrow = tid >> 3;
-  const int lsub = tid & 7;
-  // Row ids of the gathered segment are fetched one tile ahead of the rows themselves, so the
-  // dependent load (id -> row address) never sits in front of the MFMA work of a tile.
-  auto slot_id = [&](int slot) -> int {
-    int i = slot - a.n_win;
-    if (slot >= slot1 || i < 0 || i >= stop_pos) return -1;
-    return idx_b[i];
-  };
-  auto slot_src = [&](int slot, int id) -> const uint16_t* {
-    if (slot >= slot1) return nullptr;
-    if (slot < a.n_win) {
-      if (slot == subst_slot) return reinterpret_cast<const uint16_t*>(a.subst_row);
-      int r = (int)(((uint32_t)a.raw_start + (uint32_t)a.win_first + (uint32_t)slot) % (uint32_t)a.raw_cap);
-      return win_b + (int64_t)r * DK;
-    }
-    if (id < 0) return nullptr;
-    int64_t r = (int64_t)id * a.row_mul + a.row_add;
-    if (r < 0 || r >= a.n_pool) return nullptr;
-    return pool_b + r * DK;
-  };
-  u32x4_t stage[G::kLoads];
-  bool stage_valid = false;
-  auto issue_loads = [&](int tile, int id) {
-    const uint16_t* src = slot_src(slot0 + tile * kTile + lrow, id);
-    stage_valid = src != nullptr;
-    if (stage_valid) {
-      const u32x4_t* p = reinterpret_cast<const u32x4_t*>(src);
+  // ---- static part of this thread's tile loads: LDS slot P = tid + 256 j holds (row P / kSlots, chunk P % kSlots)
+  uint32_t pk[G::kPerThread];
 #pragma unroll
-      for (int j = 0; j < G::kLoads; j++) stage[j] = p[lsub + 8 * j];
-    } else {
-#pragma unroll
-      for (int j = 0; j < G::kLoads; j++) stage[j] = u32x4_t{0u, 0u, 0u, 0u};
-    }
-  };
-  auto store_stage = [&](int buf) {
-    unsigned char* dst = kbuf + buf * G::kTileBytes + lrow * G::kPitch;
-#pragma unroll
-    for (int j = 0; j < G::kLoads; j++) *reinterpret_cast<u32x4_t*>(dst + (lsub + 8 * j) * 16) = stage[j];
-    // one validity byte per wave: bit j = row 8*wave + j
-    uint64_t bal = __ballot(stage_valid);
-    if (lane == 0) {
-      uint32_t byte = 0u;
-#pragma unroll
-      for (int j = 0; j < 8; j++) byte |= (uint32_t)((bal >> (8 * j)) & 1ull) << j;
-      vmask[buf * 4 + wave] = (uint8_t)byte;
-    }
-  };
-
-  int id_next = -1;
-  if (n_tiles > 0) {
-    issue_loads(0, slot_id(slot0 + lrow));
-    id_next = slot_id(slot0 + kTile + lrow);
+  for (int j = 0; j < G::kPerThread; j++) {
+    const int P = tid + 256 * j;
+    const int row = P / G::kSlots, chunk = P % G::kSlots;
+    pk[j] = (P < G::kTileSlots && chunk != G::kSlots - 1) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
   }
+  const uint64_t zero_row = reinterpret_cast<uint64_t>(&g_zero_row[0]);
 
-  // ---- query operand: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7] per k-step
-  const int head = hb * 64 + hg * 32 + n;
-  u32x4_t qf[G::kSteps];
-  {
-    const bool live = head < a.n_heads;
-    const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)(live ? head : 0) * DK + dh * G::kHalf + 8 * g;
-    if constexpr (QDT == kQSame && !ROPE) {
-      // operands are used as stored: all loads go out back to back
-      const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
-#pragma unroll
-      for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = *reinterpret_cast<const u32x4_t*>(qp + 16 * ks);
-      if (!live) {
-#pragma unroll
-        for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
-      }
-    } else {
-      float v[G::kSteps][8];
-      if constexpr (QDT == MSPR_F32) {
-        const float* qp = reinterpret_cast<const float*>(a.q) + qoff;
-        f32x4_t raw[G::kSteps][2];
-#pragma unroll
-        for (int ks = 0; ks < G::kSteps; ks++) {
-          raw[ks][0] = *reinterpret_cast<const f32x4_t*>(qp + 16 * ks);
-          raw[ks][1] = *reinterpret_cast<const f32x4_t*>(qp + 16 * ks + 4);
+  // row pointers and validity of one tile (32 lanes of one half-wave)
+  auto fill_rows = [&](int tile, int l32, uint64_t ballot_shift) {
+    const int slot = slot0 + tile * kTile + l32;
+    uint64_t ptr = zero_row;
+    bool valid = false;
+    if (slot < slot1) {
+      if (slot < a.n_win) {
+        valid = true;
+        if (slot == subst_slot) {
+          ptr = reinterpret_cast<uint64_t>(a.subst_row);
+        } else {
+          uint32_t r = ((uint32_t)a.raw_start + (uint32_t)a.win_first + (uint32_t)slot) % (uint32_t)a.raw_cap;
+          ptr = reinterpret_cast<uint64_t>(win_b + (int64_t)r * DK);
         }
-#pragma unroll
-        for (int ks = 0; ks < G::kSteps; ks++)
-#pragma unroll
-          for (int j = 0; j < 8; j++) v[ks][j] = round_to_kdt<KDT>(raw[ks][j >> 2][j & 3]);
       } else {
-        const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
-        u32x4_t raw[G::kSteps];
-#pragma unroll
-        for (int ks = 0; ks < G::kSteps; ks++) raw[ks] = *reinterpret_cast<const u32x4_t*>(qp + 16 * ks);
-#pragma unroll
-        for (int ks = 0; ks < G::kSteps; ks++)
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            v[ks][2 * j] = unpack_lo<KDT>(raw[ks][j]);
-            v[ks][2 * j + 1] = unpack_hi<KDT>(raw[ks][j]);
-          }
-      }
-#pragma unroll
-      for (int ks = 0; ks < G::kSteps; ks++) {
-        const int d0 = dh * G::kHalf + 16 * ks + 8 * g;
-        if (ROPE && d0 >= DK - 64) {
-          // partial rope on interleaved pairs with every product and sum rounded to the element type
-#pragma unroll
-          for (int j = 0; j < 4; j++) {
-            int p = (d0 - (DK - 64)) / 2 + j;
-            float c = rope_c[p], s = rope_s[p];
-            float x0 = v[ks][2 * j], x1 = v[ks][2 * j + 1];
-            float m0 = round_to_kdt<KDT>(x0 * c), m1 = round_to_kdt<KDT>(x1 * s);
-            float m2 = round_to_kdt<KDT>(x0 * s), m3 = round_to_kdt<KDT>(x1 * c);
-            v[ks][2 * j] = round_to_kdt<KDT>(m0 - m1);
-            v[ks][2 * j + 1] = round_to_kdt<KDT>(m2 + m3);
+        const int id = ids[slot - a.n_win - id_base];
+        if (id >= 0) {
+          const int64_t r = (int64_t)id * a.row_mul + a.row_add;
+          if (r >= 0 && r < a.n_pool) {
+            valid = true;
+            ptr = reinterpret_cast<uint64_t>(pool_b + r * DK);
           }
         }
-        qf[ks] = live ? u32x4_t{pack2<KDT>(v[ks][0], v[ks][1]), pack2<KDT>(v[ks][2], v[ks][3]),
-                                pack2<KDT>(v[ks][4], v[ks][5]), pack2<KDT>(v[ks][6], v[ks][7])}
-                      : u32x4_t{0u, 0u, 0u, 0u};
       }
     }
+    rowptr[(tile % G::kBufs) * kTile + l32] = ptr;
+    const uint64_t bal = __ballot(valid);
+    if (l32 == 0) vmask[tile & 3] = (uint32_t)(bal >> ballot_shift);
+  };
+  // asynchronous loads of one tile straight into its LDS ring buffer
+  auto issue_tile = [&](int tile) {
+    const int buf = tile % G::kBufs;
+    const uint64_t* rp = rowptr + buf * kTile;
+    const uint32_t dst_lds = __builtin_amdgcn_readfirstlane(
+        (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, kbuf + buf * G::kTileBytes + wave * 1024));
+    // all row pointers first (the asm statements below are compiler barriers for memory operations)
+    uint64_t src[G::kPerThread];
+#pragma unroll
+    for (int j = 0; j < G::kPerThread; j++) {
+      const uint32_t p = pk[j];
+      const bool act = p != 0xFFFFFFFFu;
+      // lanes of the padding slot fetch a harmless duplicate so that every load is fully active
+      src[j] = rp[act ? (p >> 16) : 0] + (act ? (p & 0xFFFFu) : 0u);
+    }
+#pragma unroll
+    for (int j = 0; j < G::kPerThread; j++) {
+      if (j < G::kPerThread - 1 || wave == 0) async_load_16(src[j], dst_lds + j * 4096);
+    }
+  };
+
+  __syncthreads();  // ids visible
+  MSPR_STAMP(1);
+  if (tid < 96 && tid / 32 < n_tiles) fill_rows(tid / 32, tid & 31, (tid & 32) ? 32 : 0);
+  lds_barrier();
+  // The query loads must be complete before the first asynchronous tile load goes out: a wait left
+  // for their first use would otherwise also wait for (drain) the tile loads behind them.
+  if constexpr (QDT == MSPR_F32) {
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) asm volatile("" : "+v"(qraw32[ks][0]), "+v"(qraw32[ks][1]));
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) asm volatile("" : "+v"(qf[ks]));
   }
+  if (n_tiles > 0) issue_tile(0);
+  if (n_tiles > 1) issue_tile(1);
+  MSPR_STAMP(2);
+
+  // ---- finish the query operand (type conversion, rope) while the first tiles are in flight
+  if constexpr (QDT == kQSame && !ROPE) {
+    if (!q_live) {
+#pragma unroll
+      for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+  } else {
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) {
+      float v[8];
+      if constexpr (QDT == MSPR_F32) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = round_to_kdt<KDT>(qraw32[ks][j >> 2][j & 3]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          v[2 * j] = unpack_lo<KDT>(qf[ks][j]);
+          v[2 * j + 1] = unpack_hi<KDT>(qf[ks][j]);
+        }
+      }
+      const int d0 = dh * G::kHalf + 16 * ks + 8 * g;
+      if (ROPE && d0 >= DK - 64) {
+        // partial rope on interleaved pairs with every product and sum rounded to the element type
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          int p = (d0 - (DK - 64)) / 2 + j;
+          float c = rope_c[p], s = rope_s[p];
+          float x0 = v[2 * j], x1 = v[2 * j + 1];
+          float m0 = round_to_kdt<KDT>(x0 * c), m1 = round_to_kdt<KDT>(x1 * s);
+          float m2 = round_to_kdt<KDT>(x0 * s), m3 = round_to_kdt<KDT>(x1 * c);
+          v[2 * j] = round_to_kdt<KDT>(m0 - m1);
+          v[2 * j + 1] = round_to_kdt<KDT>(m2 + m3);
+        }
+      }
+      qf[ks] = q_live ? u32x4_t{pack2<KDT>(v[0], v[1]), pack2<KDT>(v[2], v[3]), pack2<KDT>(v[4], v[5]),
+                                 pack2<KDT>(v[6], v[7])}
+                      : u32x4_t{0u, 0u, 0u, 0u};
+    }
+  }
+  MSPR_STAMP(3);
 
   f32x16_t oacc[8];
 #pragma unroll
   for (int mt = 0; mt < 8; mt++) oacc[mt] = f32x16_t{0};
   // m_run is a lazily updated reference maximum: it only moves when a tile's maximum exceeds it by
-  // more than 8 (log2 units), so the 128 accumulator registers are rescaled a few times per kernel
-  // instead of once per tile; probabilities stay below 2^8.
+  // more than kGrow (log2 units), so the 128 accumulator registers are rescaled a few times per kernel
+  // instead of once per tile.
   float m_run = -__builtin_inff();
   float l_run = 0.0f;
 
-  if (n_tiles > 0) store_stage(0);
-  __syncthreads();
-
   // per-lane LDS offsets
-  const int a_row_off = n * G::kPitch + (dh * G::kHalf + 8 * g) * 2;                     // QK^T A operand
+  const int a_row_off = n * G::kPitch + (dh * G::kHalf + 8 * g) * 2;  // QK^T A operand
   const int tr_s = lane & 15;
   const int tr_off = (4 * g + (tr_s >> 2)) * G::kPitch + (dh * 256 + 16 * ((lane >> 4) & 1) + 4 * (tr_s & 3)) * 2;
 
   for (int t = 0; t < n_tiles; t++) {
-    const int buf = t & 1;
+    // tile t has landed once this wave's loads of it are done and every wave got here
     if (t + 1 < n_tiles) {
-      issue_loads(t + 1, id_next);
-      id_next = slot_id(slot0 + (t + 2) * kTile + lrow);
+      if (wave == 0) wait_vm_and_barrier<G::kPerThread>();
+      else wait_vm_and_barrier<G::kPerThread - 1>();
+    } else {
+      wait_vm_and_barrier<0>();
     }
+    MSPR_STAMP(4 + 6 * t);
+    if (t + 2 < n_tiles) issue_tile(t + 2);  // its ring buffer held tile t-1, which every wave has left
+    if (t + 3 < n_tiles && tid < 32) fill_rows(t + 3, tid, 0);
+    const int buf = t % G::kBufs;
     const unsigned char* kt = kbuf + buf * G::kTileBytes;
+    const uint32_t mask_all = vmask[t & 3];
 
+    MSPR_STAMP(5 + 6 * t);
     // S^T partial over this wave's half of the row width
     f32x16_t sacc = {0};
     {
@@ -352,13 +430,15 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         sacc = mfma32<KDT>(cur, qf[ks], sacc);
       }
     }
-    float* sxw = sx + (buf * 4 + wave) * (16 * 64);
+    float* sxw = sx + ((t & 1) * 4 + wave) * (16 * 64);
 #pragma unroll
     for (int c = 0; c < 4; c++)
       *reinterpret_cast<f32x4_t*>(sxw + (c * 64 + lane) * 4) =
           f32x4_t{sacc[4 * c], sacc[4 * c + 1], sacc[4 * c + 2], sacc[4 * c + 3]};
-    __syncthreads();
-    const float* sxp = sx + (buf * 4 + (wave ^ 1)) * (16 * 64);
+    MSPR_STAMP(6 + 6 * t);
+    lds_barrier();
+    MSPR_STAMP(7 + 6 * t);
+    const float* sxp = sx + ((t & 1) * 4 + (wave ^ 1)) * (16 * 64);
 #pragma unroll
     for (int c = 0; c < 4; c++) {
       f32x4_t o = *reinterpret_cast<const f32x4_t*>(sxp + (c * 64 + lane) * 4);
@@ -369,7 +449,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     }
 
     // online softmax in the log2 domain; key of register i is 8*(i/4) + 4g + i%4
-    const uint32_t mask_all = *reinterpret_cast<const uint32_t*>(vmask + buf * 4);
     float tmax = -__builtin_inff();
     if (mask_all == 0xFFFFFFFFu) {
 #pragma unroll
@@ -415,6 +494,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       pf[ks] = u32x4_t{pack2<KDT>(sacc[8 * ks], sacc[8 * ks + 1]), pack2<KDT>(sacc[8 * ks + 2], sacc[8 * ks + 3]),
                        pack2<KDT>(sacc[8 * ks + 4], sacc[8 * ks + 5]), pack2<KDT>(sacc[8 * ks + 6], sacc[8 * ks + 7])};
 
+    MSPR_STAMP(8 + 6 * t);
     // O^T += V^T . P^T ; V^T operands through the LDS transpose read of the row-major tile
 #pragma unroll
     for (int mt = 0; mt < 8; mt++) {
@@ -427,11 +507,9 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
       }
     }
-
-    if (t + 1 < n_tiles) store_stage(buf ^ 1);
-    __syncthreads();
   }
 
+  MSPR_STAMP(4 + 6 * n_tiles);
   // ---- partial results: registers go out in their native order (coalesced), stats per head
   float l_tot = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
   const int64_t part = ((int64_t)(b * a.n_hblk + hb) * a.n_splits + sp);
@@ -447,6 +525,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     ml[0] = m_run;
     ml[1] = l_tot;
   }
+  MSPR_STAMP(5 + 6 * n_tiles);
 }
 
 // Merge of the per-split partials: one workgroup per (batch, head block, wave slot, 32-column tile).
@@ -540,12 +619,15 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
 }
 
 int choose_splits(int batch_hblk, int n_keys) {
-  // enough workgroups to cover the 256 CUs, at least one 32-slot tile each, at most 64 splits
+  // enough workgroups to cover the 256 CUs, at least one 32-slot tile each, and never more gathered
+  // slots per workgroup than its LDS id table holds
   int tiles = (n_keys + kTile - 1) / kTile;
   if (tiles < 1) tiles = 1;
   int want = (256 + batch_hblk - 1) / batch_hblk;
   if (want > 32) want = 32;
   if (want > tiles) want = tiles;
+  int min_splits = (n_keys + 1023) / 1024;
+  if (want < min_splits) want = min_splits;
   if (want < 1) want = 1;
   return want;
 }
@@ -587,7 +669,9 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   int sps = (n_keys + a.n_splits - 1) / a.n_splits;
   sps = (sps + 7) / 8 * 8;
   if (sps < 8) sps = 8;
+  if (sps > 1024) sps = 1024;
   a.slots_per_split = sps;
+  MSPR_REQUIRE((int64_t)sps * a.n_splits >= n_keys, "sparse attention: too many key slots (%d)", n_keys);
   size_t need = workspace_bytes(a.batch, a.n_heads, n_keys);
   MSPR_REQUIRE(workspace && workspace_bytes_given >= need, "sparse attention: workspace of %zu bytes needed, %zu given",
                need, workspace_bytes_given);
@@ -595,6 +679,9 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   size_t parts = (size_t)a.batch * a.n_hblk * a.n_splits;
   a.ws_o = reinterpret_cast<float*>(workspace);
   a.ws_ml = a.ws_o + parts * (4 * 8 * 16 * 64);
+#ifdef MSPR_SPARSE_TRACE
+  a.trace = g_trace_buf;
+#endif
   int rc;
   if (a.rope) rc = launch_split<MSPR_F16, 512, kQSame, true>(a, st);
   else if (a.q_dtype == MSPR_F32) rc = launch_split<MSPR_F16, 512, MSPR_F32, false>(a, st);
