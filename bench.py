@@ -1,0 +1,226 @@
+#!/usr/bin/env python
+"""Benchmark of the MI355X attention hot path.
+
+One step = one DeepSeek-V4-style sparse decode attention layer at 128K context on synthetic data:
+
+    lightning-indexer scores (64 heads x 128, 32768 fp8 keys per sequence)
+      -> deterministic top-2048
+      -> sparse multi-head-latent decode attention over the 2048 gathered rows plus the last
+         128 rows of a 131072-token bf16 latent cache (576-wide K, 512-wide V, 64 heads)
+
+for a batch of 16 sequences (BASELINE configs 4 and 5 chained). Inputs are resident in HBM before
+the timed region; the step is captured in a HIP graph per buffer set and the timed loop replays
+the graphs round-robin over several buffer sets so that neither L2 nor the Infinity Cache can hold
+the streamed rows between steps.
+
+Prints ONE JSON line (see README of the driver contract): metric/value plus `roofline` for the
+dominant kernel (GPU-side duration from HIP events around that kernel on its launch stream) and
+`cpu_baseline` (the NumPy oracle on a bounded sample, on this host's cores).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+# workload constants (BASELINE configs 4 and 5)
+N_IDX_HEADS, IDX_DIM, N_KEYS, TOPK = 64, 128, 32768, 2048
+N_HEADS, K_DIM, V_DIM, N_TOKENS, WINDOW = 64, 576, 512, 131072, 128
+# algorithmic bytes per sequence: gathered rows + q + out + ids (config 5); keys + scales + q,w + ids (config 4)
+MLA_BYTES_PER_SEQ = (TOPK + WINDOW) * K_DIM * 2 + N_HEADS * K_DIM * 2 + N_HEADS * V_DIM * 2 + TOPK * 4
+IDX_BYTES_PER_SEQ = N_KEYS * IDX_DIM + N_KEYS * 4 + N_IDX_HEADS * IDX_DIM * 2 + N_IDX_HEADS * 4 + TOPK * 4
+
+
+def make_set(batch: int, dev, gen):
+    qi = torch.randn((batch, N_IDX_HEADS, IDX_DIM), device=dev, generator=gen).to(torch.bfloat16)
+    k32 = torch.randn((batch, N_KEYS, IDX_DIM), device=dev, generator=gen)
+    kscale = (k32.abs().amax(dim=-1) / 448.0).contiguous()
+    keys = (k32 / kscale[..., None]).to(torch.float8_e4m3fn)
+    del k32
+    w = torch.rand((batch, N_IDX_HEADS), device=dev, generator=gen)
+    q = torch.randn((batch, N_HEADS, K_DIM), device=dev, generator=gen).to(torch.bfloat16)
+    kv = torch.empty((batch, N_TOKENS, K_DIM), device=dev, dtype=torch.bfloat16)
+    for b in range(batch):  # chunked: the float32 intermediate of one sequence is 302 MB
+        kv[b] = torch.randn((N_TOKENS, K_DIM), device=dev, generator=gen).to(torch.bfloat16)
+    return dict(qi=qi, keys=keys, kscale=kscale, w=w, q=q, kv=kv)
+
+
+def cpu_baseline(seconds_budget: float = 15.0):
+    """The NumPy oracle on one sequence of the same step; scaled to the 16-sequence layer."""
+    from oracle import ds4
+
+    try:
+        from threadpoolctl import threadpool_limits
+    except Exception:  # pragma: no cover
+        threadpool_limits = None
+    cores = min(16, os.cpu_count() or 1)
+    rng = np.random.default_rng(0)
+    qi = ds4.round_bf16(rng.standard_normal((1, N_IDX_HEADS, IDX_DIM), dtype=np.float32))
+    k32 = rng.standard_normal((1, N_KEYS, IDX_DIM), dtype=np.float32)
+    kscale = (np.abs(k32).max(-1) / 448.0).astype(np.float32)
+    codes = ds4.e4m3_encode(k32 / kscale[..., None])
+    w = rng.uniform(0, 1, (1, N_IDX_HEADS)).astype(np.float32)
+    q = ds4.round_bf16(rng.standard_normal((1, N_HEADS, K_DIM), dtype=np.float32))
+    kv = ds4.round_bf16(rng.standard_normal((1, N_TOKENS, K_DIM), dtype=np.float32))
+    win = np.arange(N_TOKENS - WINDOW, N_TOKENS, dtype=np.int64)
+
+    def step():
+        s = ds4.indexer_scores_fp8(qi, codes, kscale, w)
+        sel = ds4.radix_select_topk(s[0].astype(np.float32), TOPK).astype(np.int64)
+        rows = np.concatenate([win, 4 * sel + 3])[None, :]
+        return ds4.sparse_mla_decode(q, kv, rows, scale=K_DIM ** -0.5)
+
+    ctx = threadpool_limits(limits=cores) if threadpool_limits else None
+    try:
+        step()
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 20 and (time.perf_counter() - t0) < seconds_budget:
+            step()
+            reps += 1
+        per_seq = (time.perf_counter() - t0) / max(reps, 1)
+    finally:
+        if ctx is not None:
+            ctx.__exit__(None, None, None)
+    return {
+        "value": per_seq * 16 * 1e6,
+        "unit": "us/layer",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{reps} repeats of one sequence (1/16 of the layer: 32768-key indexer + top-2048 + 2176-row "
+                  f"MLA decode), NumPy oracle with {cores} BLAS threads, scaled x16",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--sets", type=int, default=8, help="distinct buffer sets rotated through (cold caches)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (every box has one MI355X); rerun with --gpus 1",
+              file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        return 2
+
+    from moespresso_amd import _lib
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+    from moespresso_amd.runtime.deepseek_v4 import indexer_score_kernel as isk
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(0)
+    B, R, K, W = args.batch, max(1, args.sets), args.steps, args.warmup
+    sets = [make_set(B, dev, gen) for _ in range(R)]
+    ws = _lib.sparse_attention_workspace(B, N_HEADS, TOPK + WINDOW, dev)
+    scale = K_DIM ** -0.5
+
+    def step(s):
+        scores = isk.indexer_scores_fp8(s["qi"], s["keys"], s["kscale"], s["w"])
+        sel = isk.topk_select(scores, TOPK)
+        return iak.sparse_mla_decode(s["q"], s["kv"], sel, scale=scale, window_start=N_TOKENS - WINDOW,
+                                     window_rows=WINDOW, row_mul=4, row_add=3, workspace=ws)
+
+    # eager warm-up (also loads the code objects), then one HIP graph per buffer set
+    for s in sets:
+        step(s)
+    torch.cuda.synchronize()
+    graphs, outs = [], []
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for s in sets:
+            step(s)
+    torch.cuda.current_stream().wait_stream(side)
+    for s in sets:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            outs.append(step(s))
+        graphs.append(g)
+    torch.cuda.synchronize()
+
+    for i in range(W):
+        graphs[i % R].replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        graphs[i % R].replay()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / K * 1e3
+
+    # per-kernel GPU durations: same steps, eager, HIP events around each kernel on its launch stream
+    names = ("indexer_fp8", "topk", "sparse_split", "sparse_merge")
+    _lib.profile_enable(*names)
+    for i in range(K):
+        step(sets[i % R])
+    torch.cuda.synchronize()
+    kernel_us = {n: float(np.mean(_lib.profile_collect(n))) * 1e3 for n in names}
+    _lib.profile_enable()
+
+    split_us = kernel_us["sparse_split"]
+    achieved = MLA_BYTES_PER_SEQ * B / (split_us * 1e-6) / 1e9
+    roofline = {
+        "kernel": "sparse_attn_split_kernel<bf16,576>",
+        "bound": "hbm",
+        "achieved": round(achieved, 1),
+        "peak": HBM_PEAK_GBS,
+        "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4),
+        "traffic": None,
+        "algorithmic_bytes_per_launch": MLA_BYTES_PER_SEQ * B,
+        "kernel_us": round(split_us, 2),
+    }
+    extras = {
+        "kernel_us": {k: round(v, 2) for k, v in kernel_us.items()},
+        "indexer_fp8_GBps": round(IDX_BYTES_PER_SEQ * B / (kernel_us["indexer_fp8"] * 1e-6) / 1e9, 1),
+        "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
+        "buffer_sets": R,
+    }
+    line = {
+        "metric": "sparse decode attn us/layer @128K ctx (indexer score + top-2048 + indexed MLA decode)",
+        "value": round(ms_per_step * 1e3, 2),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"DS4-style sparse decode attention layer, batch {B}: 64x128 indexer over 32768 fp8 keys, "
+                        f"top-2048, MLA decode over 2048 gathered + 128 window rows of a 131072-token bf16 cache "
+                        f"(576-wide K, 512-wide V, 64 heads)",
+            "batch": B,
+            "context": N_TOKENS,
+        },
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
+        "extras": extras,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
