@@ -142,6 +142,33 @@ int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, c
                            int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
                            float scale, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------ Qwen/Ornith GQA attention, 8-bit KV */
+
+/* Workspace bytes of the two Q8 decode entry points below. */
+size_t mspr_sdpa_decode_q8_workspace_bytes(int batch, int n_kv_heads, int64_t n_keys);
+
+/* One-token GQA decode attention over an MLX affine 8-bit KV cache, dequantised in-kernel.
+ * Replaces mlx_kquant.sdpa_decode_q8 as called from runtime/qwen/full_attention.py:323
+ * (third-party Metal operator, not vendored; arguments follow that call site).
+ * queries: f32 [batch,n_q_heads,1,256]; k_wq/v_wq: uint32 [batch,n_kv_heads,n_keys,64] (four codes
+ * per word, lowest byte first); scales and biases: [batch,n_kv_heads,n_keys,4] of sb_dtype,
+ * value = code*scale + bias per 64 elements; out: f32 [batch,n_q_heads,1,256].
+ * group_size must be 64 and bits 8; n_q_heads/n_kv_heads <= 16. */
+int mspr_sdpa_decode_q8(const void* queries, int q_dtype, const void* k_wq, const void* k_scales,
+                        const void* k_biases, const void* v_wq, const void* v_scales,
+                        const void* v_biases, int sb_dtype, int batch, int n_q_heads, int n_kv_heads,
+                        int head_dim, int64_t n_keys, float scale, int group_size, int bits, void* out,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Extension (BASELINE config 3): the same decode over a Q8_0 cache — int8 codes
+ * [batch,n_kv_heads,n_keys,256] with one float16 scale per 32 elements
+ * [batch,n_kv_heads,n_keys,8], value = code*scale. queries/out: [batch,n_q_heads,256] of q_dtype
+ * (f32|f16|bf16). */
+int mspr_sdpa_decode_q8_0(const void* queries, int q_dtype, const void* k_codes, const void* k_scales,
+                          const void* v_codes, const void* v_scales, int batch, int n_q_heads,
+                          int n_kv_heads, int head_dim, int64_t n_keys, float scale, void* out,
+                          void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ measurement */
 
 /* Per-kernel GPU timing for benchmarks. Bit k of kernel_mask brackets every later launch of kernel

@@ -46,6 +46,13 @@ SIGNATURES = {
     "mspr_sparse_mla_decode": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int64, c_int,
                 c_int, c_int, c_int64, c_int, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mspr_sdpa_decode_q8_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),
+    "mspr_sdpa_decode_q8": (
+        c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mspr_sdpa_decode_q8_0": (
+        c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int64,
+                c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_profile_enable": (c_int, [c_int]),
     "mspr_profile_collect": (c_int, [c_int, c_void_p, c_int]),
 }
@@ -74,6 +81,14 @@ def sparse_attention_workspace(batch: int, n_heads: int, n_keys: int, device) ->
     """Scratch tensor for the gathered-attention entry points (split partials)."""
     nbytes = int(lib().mspr_sparse_attention_workspace_bytes(int(batch), int(n_heads), int(n_keys)))
     return torch.empty((max(nbytes, 16) + 3) // 4, dtype=torch.float32, device=device)
+
+
+
+def q8_decode_workspace(batch: int, n_kv_heads: int, n_keys: int, device) -> torch.Tensor:
+    """Scratch tensor for the Q8 decode entry points (per-range partials)."""
+    nbytes = int(lib().mspr_sdpa_decode_q8_workspace_bytes(int(batch), int(n_kv_heads), int(n_keys)))
+    return torch.empty((max(nbytes, 16) + 3) // 4, dtype=torch.float32, device=device)
+
 
 _LIB = None
 

@@ -1,0 +1,125 @@
+"""8-bit-KV attention operators for the Qwen/Ornith full-attention layers on MI355X.
+
+The reference calls two operators of the third-party ``mlx_kquant`` Metal package from
+``src/moespresso/runtime/qwen/full_attention.py``: ``sdpa_decode_q8`` (:323) for one-token decode
+and ``sdpa_fa_prefill_q8`` (:372) for chunked causal prefill over a quantised prefix. This module
+provides operators of the same names and argument order on HIP tensors. The Metal tuning keywords
+of the reference call sites (``splits``, ``stage``, ``compute``, ``tile_c``, ``bq``, ``bk``,
+``dimension_parallel_merge``) are accepted and ignored: tiling and the split count are chosen for
+the 256 compute units of the device by the library.
+
+Cache layout (the MLX affine quantiser, ``mx.quantize(x, group_size=64, bits=8)``): ``wq`` uint32
+``[B, Hkv, N, D/4]`` with four codes per word (lowest byte first), ``scales`` and ``biases``
+``[B, Hkv, N, D/64]``; value = code * scale + bias.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from moespresso_amd import _lib
+
+_HEAD_DIM = 256
+
+
+def _check_q8_triplet(name, wq, scales, biases, batch, n_keys=None):
+    if wq.ndim != 4 or scales.ndim != 4 or biases.ndim != 4:
+        raise ValueError(f"{name} quantized tensors must be rank-4 [B, Hkv, N, *]")
+    if wq.dtype != torch.uint32 and wq.dtype != torch.int32 and wq.dtype != torch.uint8:
+        raise ValueError(f"{name} codes must be uint32 words (or their uint8 view)")
+    width = int(wq.shape[-1]) * (4 if wq.dtype != torch.uint8 else 1)
+    if width != _HEAD_DIM:
+        raise ValueError("q8 attention requires head_dim=256")
+    if int(scales.shape[-1]) != _HEAD_DIM // 64 or tuple(scales.shape) != tuple(biases.shape):
+        raise ValueError(f"{name} scales and biases must be [B, Hkv, N, 4] (group_size=64)")
+    if scales.dtype != biases.dtype or scales.dtype not in _lib.DTYPE_CODE:
+        raise ValueError(f"{name} scales and biases must share a float32/float16/bfloat16 dtype")
+    if tuple(wq.shape[:3]) != tuple(scales.shape[:3]) or int(wq.shape[0]) != batch:
+        raise ValueError(f"{name} codes, scales and biases disagree on [B, Hkv, N]")
+    if n_keys is not None and int(wq.shape[2]) != n_keys:
+        raise ValueError("keys and values disagree on the number of cached tokens")
+
+
+def sdpa_decode_q8(queries, k_wq, k_scales, k_biases, v_wq, v_scales, v_biases, scale, *, group_size: int = 64,
+                   bits: int = 8, workspace=None, **_tuning):
+    """One-token GQA attention over an affine 8-bit KV cache (reference call site full_attention.py:323).
+
+    Args:
+        queries: float32 ``[B, Hq, 1, 256]`` (already rotated).
+        k_wq, k_scales, k_biases / v_wq, v_scales, v_biases: the quantised cache of ``N`` tokens.
+        scale: softmax scale.
+
+    Returns:
+        float32 ``[B, Hq, 1, 256]``.
+    """
+    if group_size != 64 or bits != 8:
+        raise ValueError("sdpa_decode_q8 supports group_size=64, bits=8 only")
+    if queries.ndim != 4 or int(queries.shape[2]) != 1:
+        raise ValueError("queries must be [B, Hq, 1, D] (single-token decode)")
+    if int(queries.shape[3]) != _HEAD_DIM:
+        raise ValueError("q8 attention requires head_dim=256")
+    if queries.dtype != torch.float32:
+        raise ValueError("queries must be float32")
+    B, Hq = int(queries.shape[0]), int(queries.shape[1])
+    _check_q8_triplet("key", k_wq, k_scales, k_biases, B)
+    N = int(k_wq.shape[2])
+    _check_q8_triplet("value", v_wq, v_scales, v_biases, B, N)
+    Hkv = int(k_wq.shape[1])
+    if int(v_wq.shape[1]) != Hkv or Hq % Hkv != 0 or Hq // Hkv > 16:
+        raise ValueError("query heads must be a multiple (at most 16x) of the KV heads")
+    if k_scales.dtype != v_scales.dtype:
+        raise ValueError("key and value scales must share a dtype")
+    if N < 1:
+        raise ValueError("the cache must hold at least one token")
+    _lib.require_device(queries, k_wq, k_scales, k_biases, v_wq, v_scales, v_biases)
+    tensors = [t.contiguous() for t in (queries, k_wq, k_scales, k_biases, v_wq, v_scales, v_biases)]
+    q, kw, ks, kb, vw, vs, vb = tensors
+    out = torch.empty_like(q)
+    if workspace is None:
+        workspace = _lib.q8_decode_workspace(B, Hkv, N, q.device)
+    _lib.check(_lib.lib().mspr_sdpa_decode_q8(
+        _lib.ptr(q), _lib.DTYPE_CODE[q.dtype], _lib.ptr(kw), _lib.ptr(ks), _lib.ptr(kb), _lib.ptr(vw), _lib.ptr(vs),
+        _lib.ptr(vb), _lib.DTYPE_CODE[ks.dtype], B, Hq, Hkv, _HEAD_DIM, N, float(scale), 64, 8, _lib.ptr(out),
+        _lib.ptr(workspace), workspace.numel() * workspace.element_size(), _lib.stream_ptr()), "sdpa_decode_q8")
+    return out
+
+
+def sdpa_decode_q8_0(queries, k_codes, k_scales, v_codes, v_scales, scale, *, workspace=None):
+    """One-token GQA attention over a Q8_0 KV cache (int8 codes, one float16 scale per 32 elements).
+
+    Args:
+        queries: ``[B, Hq, 256]`` float32, float16 or bfloat16.
+        k_codes, v_codes: int8 ``[B, Hkv, N, 256]``; k_scales, v_scales: float16 ``[B, Hkv, N, 8]``.
+
+    Returns:
+        ``[B, Hq, 256]`` in the dtype of ``queries``.
+    """
+    if queries.ndim != 3 or int(queries.shape[2]) != _HEAD_DIM:
+        raise ValueError("queries must be [B, Hq, 256]")
+    if queries.dtype not in _lib.DTYPE_CODE:
+        raise ValueError("queries must be float32, float16 or bfloat16")
+    B, Hq = int(queries.shape[0]), int(queries.shape[1])
+    for name, c, s in (("key", k_codes, k_scales), ("value", v_codes, v_scales)):
+        if c.ndim != 4 or c.dtype != torch.int8 or int(c.shape[3]) != _HEAD_DIM:
+            raise ValueError(f"{name} codes must be int8 [B, Hkv, N, 256]")
+        if s.dtype != torch.float16 or tuple(s.shape) != tuple(c.shape[:3]) + (_HEAD_DIM // 32,):
+            raise ValueError(f"{name} scales must be float16 [B, Hkv, N, 8]")
+        if int(c.shape[0]) != B:
+            raise ValueError(f"{name} cache batch must match queries")
+    if tuple(k_codes.shape) != tuple(v_codes.shape):
+        raise ValueError("keys and values disagree on the number of cached tokens")
+    Hkv, N = int(k_codes.shape[1]), int(k_codes.shape[2])
+    if Hq % Hkv != 0 or Hq // Hkv > 16:
+        raise ValueError("query heads must be a multiple (at most 16x) of the KV heads")
+    if N < 1:
+        raise ValueError("the cache must hold at least one token")
+    _lib.require_device(queries, k_codes, k_scales, v_codes, v_scales)
+    q, kc, ks, vc, vs = [t.contiguous() for t in (queries, k_codes, k_scales, v_codes, v_scales)]
+    out = torch.empty_like(q)
+    if workspace is None:
+        workspace = _lib.q8_decode_workspace(B, Hkv, N, q.device)
+    _lib.check(_lib.lib().mspr_sdpa_decode_q8_0(
+        _lib.ptr(q), _lib.DTYPE_CODE[q.dtype], _lib.ptr(kc), _lib.ptr(ks), _lib.ptr(vc), _lib.ptr(vs), B, Hq, Hkv,
+        _HEAD_DIM, N, float(scale), _lib.ptr(out), _lib.ptr(workspace),
+        workspace.numel() * workspace.element_size(), _lib.stream_ptr()), "sdpa_decode_q8_0")
+    return out
