@@ -169,6 +169,16 @@ int mspr_sdpa_decode_q8_0(const void* queries, int q_dtype, const void* k_codes,
                           int n_kv_heads, int head_dim, int64_t n_keys, float scale, void* out,
                           void* workspace, size_t workspace_bytes, void* stream);
 
+/* Causal chunked-prefill GQA attention over a dense 16-bit KV cache that already holds the chunk:
+ * query row i (position past_len + i) attends keys [0, past_len + i].
+ * Stands in for mx.fast.scaled_dot_product_attention(mask="causal") over the fetched cache, the
+ * composed prefill route of runtime/qwen/full_attention.py:399-409, at BASELINE config 2.
+ * q/out: [batch,n_q_heads,q_len,256] of dtype (f16|bf16); k, v: [batch,n_kv_heads,kv_rows,256]
+ * same dtype, rows [0, past_len+q_len) valid; n_q_heads/n_kv_heads in {1,2,4,8}. */
+int mspr_flash_prefill(const void* q, const void* k, const void* v, int dtype, int batch, int n_q_heads,
+                       int n_kv_heads, int head_dim, int q_len, int64_t past_len, int64_t kv_rows,
+                       float scale, void* out, void* stream);
+
 /* ------------------------------------------------------------------ measurement */
 
 /* Per-kernel GPU timing for benchmarks. Bit k of kernel_mask brackets every later launch of kernel

@@ -53,6 +53,9 @@ SIGNATURES = {
     "mspr_sdpa_decode_q8_0": (
         c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int64,
                 c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mspr_flash_prefill": (
+        c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_float,
+                c_void_p, c_void_p]),
     "mspr_profile_enable": (c_int, [c_int]),
     "mspr_profile_collect": (c_int, [c_int, c_void_p, c_int]),
 }

@@ -123,3 +123,43 @@ def sdpa_decode_q8_0(queries, k_codes, k_scales, v_codes, v_scales, scale, *, wo
         _HEAD_DIM, N, float(scale), _lib.ptr(out), _lib.ptr(workspace),
         workspace.numel() * workspace.element_size(), _lib.stream_ptr()), "sdpa_decode_q8_0")
     return out
+
+
+def flash_prefill(queries, keys, values, scale, *, past_len: int):
+    """Causal chunked-prefill GQA attention over a dense 16-bit cache that already holds the chunk.
+
+    Query row ``i`` sits at position ``past_len + i`` and attends keys ``[0, past_len + i]``: the
+    arithmetic of the reference's composed prefill route (``scaled_dot_product_attention`` with
+    ``mask="causal"`` over the fetched cache, full_attention.py:399-409).
+
+    Args:
+        queries: ``[B, Hq, L, 256]`` float16 or bfloat16.
+        keys, values: ``[B, Hkv, rows, 256]`` of the same dtype, ``rows >= past_len + L``.
+
+    Returns:
+        ``[B, Hq, L, 256]`` in the dtype of ``queries``.
+    """
+    if queries.ndim != 4 or keys.ndim != 4 or values.ndim != 4:
+        raise ValueError("queries, keys and values must be rank-4 [B, H, T, D]")
+    if int(queries.shape[3]) != _HEAD_DIM or int(keys.shape[3]) != _HEAD_DIM or int(values.shape[3]) != _HEAD_DIM:
+        raise ValueError("flash prefill requires head_dim=256")
+    if queries.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("queries must be float16 or bfloat16")
+    if keys.dtype != queries.dtype or values.dtype != queries.dtype:
+        raise ValueError("keys and values must have the dtype of queries")
+    if tuple(keys.shape) != tuple(values.shape) or int(keys.shape[0]) != int(queries.shape[0]):
+        raise ValueError("keys and values must share a shape and the batch of queries")
+    B, Hq, L = int(queries.shape[0]), int(queries.shape[1]), int(queries.shape[2])
+    Hkv, rows = int(keys.shape[1]), int(keys.shape[2])
+    if Hq % Hkv != 0 or Hq // Hkv not in (1, 2, 4, 8):
+        raise ValueError("query heads per KV head must be 1, 2, 4 or 8")
+    past_len = int(past_len)
+    if L < 1 or past_len < 0 or past_len + L > rows:
+        raise ValueError("need q_len >= 1, past_len >= 0 and past_len + q_len <= cache rows")
+    _lib.require_device(queries, keys, values)
+    q, k, v = queries.contiguous(), keys.contiguous(), values.contiguous()
+    out = torch.empty_like(q)
+    _lib.check(_lib.lib().mspr_flash_prefill(
+        _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.DTYPE_CODE[q.dtype], B, Hq, Hkv, _HEAD_DIM, L, past_len, rows,
+        float(scale), _lib.ptr(out), _lib.stream_ptr()), "flash_prefill")
+    return out
