@@ -179,6 +179,25 @@ int mspr_flash_prefill(const void* q, const void* k, const void* v, int dtype, i
                        int n_kv_heads, int head_dim, int q_len, int64_t past_len, int64_t kv_rows,
                        float scale, void* out, void* stream);
 
+/* Workspace bytes of mspr_sdpa_fa_prefill_q8 (float16 copies of the chunk's own K/V rows). */
+size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_kv_heads, int q_len, int64_t past_len);
+
+/* Causal flash prefill over an affine 8-bit prefix plus the dense chunk itself: query row i attends
+ * every prefix key and chunk keys [0, i].
+ * Replaces mlx_kquant.sdpa_fa_prefill_q8 as called from runtime/qwen/full_attention.py:372
+ * (third-party Metal operator, not vendored; arguments follow that call site and the helper at
+ * tests/test_qwen_flash_prefill_attention.py:361-375).
+ * queries/out: f32 [batch,n_q_heads,q_len,256]; pk_wq/pv_wq: uint32 [batch,n_kv_heads,past_len,64];
+ * their scales and biases: [batch,n_kv_heads,past_len,4] of sb_dtype; self_k/self_v:
+ * [batch,n_kv_heads,q_len,256] of self_dtype (already passed through the 8-bit round trip by the
+ * caller). past_len may be 0 (the prefix pointers are then ignored). */
+int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, const void* pk_scales,
+                            const void* pk_biases, const void* pv_wq, const void* pv_scales,
+                            const void* pv_biases, int sb_dtype, const void* self_k, const void* self_v,
+                            int self_dtype, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                            int q_len, int64_t past_len, float scale, int group_size, int bits, void* out,
+                            void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------------------------ measurement */
 
 /* Per-kernel GPU timing for benchmarks. Bit k of kernel_mask brackets every later launch of kernel

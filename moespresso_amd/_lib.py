@@ -56,6 +56,11 @@ SIGNATURES = {
     "mspr_flash_prefill": (
         c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_float,
                 c_void_p, c_void_p]),
+    "mspr_sdpa_fa_prefill_q8_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int64]),
+    "mspr_sdpa_fa_prefill_q8": (
+        c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p, c_void_p,
+                c_size_t, c_void_p]),
     "mspr_profile_enable": (c_int, [c_int]),
     "mspr_profile_collect": (c_int, [c_int, c_void_p, c_int]),
 }

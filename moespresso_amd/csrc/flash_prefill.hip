@@ -37,7 +37,46 @@ struct PrefillArgs {
   float scale_log2;
   int rep_shift;    // log2(query heads per KV head), 0..3
   int q_blocks;     // workgroups along the query axis
+  // quantised-prefix form only: tiles [0, q8_tiles) come from the affine 8-bit prefix below, the rest
+  // from k / v, which then hold float16 rows for keys [32 q8_tiles, past_len + q_len)
+  int q8_tiles;
+  const void* pk_wq;  // [B, Hkv, past_len, 256] codes
+  const void* pk_s;   // [B, Hkv, past_len, 4]
+  const void* pk_b;
+  const void* pv_wq;
+  const void* pv_s;
+  const void* pv_b;
 };
+
+typedef __attribute__((ext_vector_type(2))) _Float16 h2_t;
+__device__ __forceinline__ uint32_t h2_bits(h2_t v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ h2_t bits_h2(uint32_t v) { return __builtin_bit_cast(h2_t, v); }
+// raw affine scale / bias bits to a packed float16 pair
+template <int SDT>
+__device__ __forceinline__ h2_t sb_to_h2(uint32_t bits) {
+  _Float16 h;
+  if constexpr (SDT == MSPR_F32) h = (_Float16)__builtin_bit_cast(float, bits);
+  else if constexpr (SDT == MSPR_F16) h = __builtin_bit_cast(_Float16, (uint16_t)bits);
+  else h = (_Float16)__builtin_bit_cast(float, bits << 16);
+  return h2_t{h, h};
+}
+// 16 unsigned 8-bit codes -> 16 float16 values code * scale + bias (two 16-byte pieces)
+__device__ __forceinline__ void dequant16(u32x4_t c, h2_t sc, h2_t bi, u32x4_t& p0, u32x4_t& p1) {
+  const h2_t k1024 = {(_Float16)1024.0f, (_Float16)1024.0f};
+#pragma unroll
+  for (int w = 0; w < 4; w++) {
+    // byte b becomes the float16 with bits 0x6400 | b = 1024 + b, exactly
+    h2_t lo = (bits_h2(__builtin_amdgcn_perm(0x64646464u, c[w], 0x04010400u)) - k1024) * sc + bi;
+    h2_t hi = (bits_h2(__builtin_amdgcn_perm(0x64646464u, c[w], 0x04030402u)) - k1024) * sc + bi;
+    if (w < 2) {
+      p0[2 * w] = h2_bits(lo);
+      p0[2 * w + 1] = h2_bits(hi);
+    } else {
+      p1[2 * (w - 2)] = h2_bits(lo);
+      p1[2 * (w - 2) + 1] = h2_bits(hi);
+    }
+  }
+}
 
 template <int KDT>
 __device__ __forceinline__ f32x16_t mfma32(u32x4_t a, u32x4_t b, f32x16_t c) {
@@ -75,7 +114,9 @@ __device__ __forceinline__ void async_load_16(uint64_t base, uint32_t offset, ui
 // swizzle of the 16-byte pieces of a tile row: piece p of row r sits at slot (p & 16) | ((p ^ f(r)) & 15)
 __device__ __forceinline__ int swz(int r) { return ((r & 7) << 1) | ((r >> 3) & 1); }
 
-template <int KDT>
+// Q8 = false: k / v are the whole 16-bit cache, q / out have its element type.
+// Q8 = true (KDT float16): float32 q / out, quantised prefix + float16 tail rows (see PrefillArgs).
+template <int KDT, bool Q8, int SDT>
 __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int tid = threadIdx.x;
@@ -114,9 +155,11 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   const uint32_t lds0 = (uint32_t)(uintptr_t)MSPR_LDS_PTR(unsigned char, lds);
   const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(lds0) + wave * 1024;
   const int n_keys = (int)(past + a.q_len);  // keys that exist
-  auto issue_tile = [&](int t, int slot) {
+  const int t1 = Q8 ? a.q8_tiles : 0;        // first tile served from k / v; their row 0 is key 32 t1
+  auto issue_tile = [&](int t_abs, int slot) {
     // rows past the last key (only in the last tile) are masked by the causal rule; read the last key instead
-    const int last = n_keys - 1 - t * kTile;
+    const int t = t_abs - t1;
+    const int last = n_keys - 1 - t_abs * kTile;
     const uint32_t o0 = (uint32_t)((c_row < last ? c_row : last) * kRowBytes + c_piece * 16);
     const uint32_t o1 = (uint32_t)((c_row + 16 < last ? c_row + 16 : last) * kRowBytes + c_piece * 16);
     const uint64_t kt = (uint64_t)(kbase + (int64_t)t * kTileBytes);
@@ -134,18 +177,31 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
     int qrow = q0 + n;
     if (qrow > a.q_len - 1) qrow = a.q_len - 1;
     if (qrow < 0) qrow = 0;
-    const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(
-        reinterpret_cast<const unsigned char*>(a.q) + (((int64_t)b * a.n_q_heads + head) * a.q_len + qrow) * kRowBytes +
-        16 * g);
+    const int64_t qoff = (((int64_t)b * a.n_q_heads + head) * a.q_len + qrow) * kD + 8 * g;
+    if constexpr (!Q8) {
+      const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(a.q) + qoff);
 #pragma unroll
-    for (int s = 0; s < 16; s++) qf[s] = qp[2 * s];
+      for (int s = 0; s < 16; s++) qf[s] = qp[2 * s];
+    } else {
+      const f32x4_t* qp = reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(a.q) + qoff);
+#pragma unroll
+      for (int s0 = 0; s0 < 16; s0 += 4) {
+        f32x4_t raw[8];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          raw[2 * j] = qp[4 * (s0 + j)];
+          raw[2 * j + 1] = qp[4 * (s0 + j) + 1];
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          qf[s0 + j] = u32x4_t{pack2<KDT>(raw[2 * j][0], raw[2 * j][1]), pack2<KDT>(raw[2 * j][2], raw[2 * j][3]),
+                               pack2<KDT>(raw[2 * j + 1][0], raw[2 * j + 1][1]),
+                               pack2<KDT>(raw[2 * j + 1][2], raw[2 * j + 1][3])};
+      }
+    }
 #pragma unroll
     for (int s = 0; s < 16; s++) asm volatile("" : "+v"(qf[s]));  // complete before the first asynchronous copy
   }
-
-  // every wave issues its share of every tile (clamped past the end), so waits are static counts
-  issue_tile(0, 0);
-  issue_tile(n_tiles > 1 ? 1 : 0, 1);
 
   f32x16_t oacc[8];
 #pragma unroll
@@ -167,15 +223,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   const int my_last_key = past + q0 + 31;  // last key any query of this wave may see
   const int qpos = past + q0 + n;
 
-  for (int t = 0; t < n_tiles; t++) {
-    // tile t has landed once this wave's copies of it are done (4 newer ones may be in flight) and
-    // every wave got here; the ring slot of tile t-1 is free after the barrier
-    wait_vm_and_barrier<4>();
-    issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t + 2) % kBufs);  // past the end: a harmless re-read
-    const int key0 = t * kTile;
-    if (key0 > my_last_key) continue;  // wave-uniform: this wave's queries see none of the tile
-    const unsigned char* st = lds + (t % kBufs) * kStageBytes;
-
+  auto compute_tile = [&](const unsigned char* st, int key0) {
     // S^T = K . Q^T
     f32x16_t sacc = {0};
     {
@@ -249,6 +297,80 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
         oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
       }
     }
+  };
+
+  if constexpr (Q8) {
+    // ---- quantised prefix: tile t+1 is unpacked from registers into the other LDS slot at the top of
+    //      step t while the raw bytes of tile t+2 are already on their way
+    if (t1 > 0) {
+      const int s_row = tid >> 4;   // tile row staged by this thread
+      const int s_pp = tid & 15;    // its 16 elements: [16 s_pp, +16), scale group s_pp / 4
+      const int64_t row0 = ((int64_t)b * a.n_kv_heads + kvh) * past;
+      const uint8_t* kc = reinterpret_cast<const uint8_t*>(a.pk_wq) + row0 * kD + 16 * s_pp;
+      const uint8_t* vc = reinterpret_cast<const uint8_t*>(a.pv_wq) + row0 * kD + 16 * s_pp;
+      constexpr int kSB = SDT == MSPR_F32 ? 4 : 2;
+      const uint8_t* ks = reinterpret_cast<const uint8_t*>(a.pk_s) + (row0 * 4 + (s_pp >> 2)) * kSB;
+      const uint8_t* kb = reinterpret_cast<const uint8_t*>(a.pk_b) + (row0 * 4 + (s_pp >> 2)) * kSB;
+      const uint8_t* vs = reinterpret_cast<const uint8_t*>(a.pv_s) + (row0 * 4 + (s_pp >> 2)) * kSB;
+      const uint8_t* vb = reinterpret_cast<const uint8_t*>(a.pv_b) + (row0 * 4 + (s_pp >> 2)) * kSB;
+      const int f = swz(s_row);
+      const int w_off0 = s_row * kRowBytes + 16 * (((2 * s_pp) & 16) | (((2 * s_pp) ^ f) & 15));
+      const int w_off1 = s_row * kRowBytes + 16 * (((2 * s_pp + 1) & 16) | (((2 * s_pp + 1) ^ f) & 15));
+      u32x4_t rk, rv;
+      uint32_t rs[4];
+      auto load_raw = [&](int t) {
+        const int64_t key = (int64_t)t * kTile + s_row;  // < past: only whole prefix tiles come through here
+        rk = *reinterpret_cast<const u32x4_t*>(kc + key * kD);
+        rv = *reinterpret_cast<const u32x4_t*>(vc + key * kD);
+        if constexpr (SDT == MSPR_F32) {
+          rs[0] = *reinterpret_cast<const uint32_t*>(ks + key * 16);
+          rs[1] = *reinterpret_cast<const uint32_t*>(kb + key * 16);
+          rs[2] = *reinterpret_cast<const uint32_t*>(vs + key * 16);
+          rs[3] = *reinterpret_cast<const uint32_t*>(vb + key * 16);
+        } else {
+          rs[0] = *reinterpret_cast<const uint16_t*>(ks + key * 8);
+          rs[1] = *reinterpret_cast<const uint16_t*>(kb + key * 8);
+          rs[2] = *reinterpret_cast<const uint16_t*>(vs + key * 8);
+          rs[3] = *reinterpret_cast<const uint16_t*>(vb + key * 8);
+        }
+      };
+      auto unpack_to = [&](int slot) {
+        unsigned char* st = lds + slot * kStageBytes;
+        u32x4_t p0, p1;
+        dequant16(rk, sb_to_h2<SDT>(rs[0]), sb_to_h2<SDT>(rs[1]), p0, p1);
+        *reinterpret_cast<u32x4_t*>(st + w_off0) = p0;
+        *reinterpret_cast<u32x4_t*>(st + w_off1) = p1;
+        dequant16(rv, sb_to_h2<SDT>(rs[2]), sb_to_h2<SDT>(rs[3]), p0, p1);
+        *reinterpret_cast<u32x4_t*>(st + kTileBytes + w_off0) = p0;
+        *reinterpret_cast<u32x4_t*>(st + kTileBytes + w_off1) = p1;
+      };
+      load_raw(0);
+      unpack_to(0);
+      if (t1 > 1) load_raw(1);
+      for (int t = 0; t < t1; t++) {
+        __syncthreads();  // tile t is complete in LDS; every wave has left tile t-1
+        if (t + 1 < t1) {
+          unpack_to((t + 1) & 1);
+          if (t + 2 < t1) load_raw(t + 2);
+        }
+        compute_tile(lds + (t & 1) * kStageBytes, t * kTile);
+      }
+      __syncthreads();  // every wave has left the last prefix tile before the ring below reuses the slots
+    }
+  }
+
+  // ---- dense tiles through the asynchronous ring: every wave issues its share of every tile
+  //      (clamped past the end), so the waits are static counts
+  issue_tile(t1, 0);
+  issue_tile(t1 + 1 < n_tiles ? t1 + 1 : n_tiles - 1, 1);
+  for (int t = t1; t < n_tiles; t++) {
+    // tile t has landed once this wave's copies of it are done (4 newer ones may be in flight) and
+    // every wave got here; the ring slot of tile t-1 is free after the barrier
+    wait_vm_and_barrier<4>();
+    issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - t1 + 2) % kBufs);  // past the end: a harmless re-read
+    const int key0 = t * kTile;
+    if (key0 > my_last_key) continue;  // wave-uniform: this wave's queries see none of the tile
+    compute_tile(lds + ((t - t1) % kBufs) * kStageBytes, key0);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped trailing copies must not outlive the workgroup's LDS
 
@@ -256,24 +378,65 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   const float l_tot = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
   if (q0 + n < a.q_len) {
-    unsigned char* op = reinterpret_cast<unsigned char*>(a.out) +
-                        (((int64_t)b * a.n_q_heads + head) * a.q_len + q0 + n) * kRowBytes;
+    const int64_t ooff = (((int64_t)b * a.n_q_heads + head) * a.q_len + q0 + n) * kD;
 #pragma unroll
     for (int mt = 0; mt < 8; mt++)
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        u32x2_t w = {pack2<KDT>(oacc[mt][4 * c] * inv, oacc[mt][4 * c + 1] * inv),
-                     pack2<KDT>(oacc[mt][4 * c + 2] * inv, oacc[mt][4 * c + 3] * inv)};
-        *reinterpret_cast<u32x2_t*>(op + (32 * mt + 8 * c + 4 * g) * 2) = w;
+        if constexpr (Q8) {
+          *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.out) + ooff + 32 * mt + 8 * c + 4 * g) =
+              f32x4_t{oacc[mt][4 * c] * inv, oacc[mt][4 * c + 1] * inv, oacc[mt][4 * c + 2] * inv,
+                      oacc[mt][4 * c + 3] * inv};
+        } else {
+          u32x2_t w = {pack2<KDT>(oacc[mt][4 * c] * inv, oacc[mt][4 * c + 1] * inv),
+                       pack2<KDT>(oacc[mt][4 * c + 2] * inv, oacc[mt][4 * c + 3] * inv)};
+          *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + ooff + 32 * mt + 8 * c + 4 * g) = w;
+        }
       }
   }
 }
 
-template <int KDT>
+// Float16 tail rows of the quantised-prefix form: key 32 q8_tiles + j for j in [0, tail_rows), the
+// last (past_len % 32) prefix rows dequantised, then the chunk's own rows converted.
+template <int SDT>
+__global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, const void* self_k, const void* self_v,
+                                                              int self_dtype, uint16_t* tail_k, uint16_t* tail_v,
+                                                              int tail_rows) {
+  const int d = threadIdx.x;
+  const int j = blockIdx.x;
+  const int kvh = blockIdx.y;
+  const int b = blockIdx.z;
+  const int64_t bh = (int64_t)b * a.n_kv_heads + kvh;
+  const int64_t key = (int64_t)a.q8_tiles * kTile + j;
+  float kx, vx;
+  if (key < a.past_len) {
+    const int64_t row = bh * a.past_len + key;
+    const float ks = load_as_f32<SDT>(a.pk_s, row * 4 + d / 64), kb = load_as_f32<SDT>(a.pk_b, row * 4 + d / 64);
+    const float vs = load_as_f32<SDT>(a.pv_s, row * 4 + d / 64), vb = load_as_f32<SDT>(a.pv_b, row * 4 + d / 64);
+    kx = (float)reinterpret_cast<const uint8_t*>(a.pk_wq)[row * kD + d] * ks + kb;
+    vx = (float)reinterpret_cast<const uint8_t*>(a.pv_wq)[row * kD + d] * vs + vb;
+  } else {
+    const int64_t off = (bh * a.q_len + (key - a.past_len)) * kD + d;
+    if (self_dtype == MSPR_F32) {
+      kx = load_as_f32<MSPR_F32>(self_k, off);
+      vx = load_as_f32<MSPR_F32>(self_v, off);
+    } else if (self_dtype == MSPR_F16) {
+      kx = load_as_f32<MSPR_F16>(self_k, off);
+      vx = load_as_f32<MSPR_F16>(self_v, off);
+    } else {
+      kx = load_as_f32<MSPR_BF16>(self_k, off);
+      vx = load_as_f32<MSPR_BF16>(self_v, off);
+    }
+  }
+  tail_k[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(kx);
+  tail_v[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(vx);
+}
+
+template <int KDT, bool Q8, int SDT>
 int prefill_launch(const PrefillArgs& a, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&flash_prefill_kernel<KDT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&flash_prefill_kernel<KDT, Q8, SDT>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess) {
       mspr_set_error("flash_prefill: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
@@ -284,7 +447,7 @@ int prefill_launch(const PrefillArgs& a, hipStream_t st) {
   dim3 grid((unsigned)(a.q_blocks * a.n_kv_heads * a.batch)), block(kThreads);
   {
     MsprProfScope prof(MSPR_K_FLASH_PREFILL, st);
-    flash_prefill_kernel<KDT><<<grid, block, kLdsBytes, st>>>(a);
+    flash_prefill_kernel<KDT, Q8, SDT><<<grid, block, kLdsBytes, st>>>(a);
   }
   MSPR_CHECK_LAUNCH("flash_prefill");
   return MSPR_OK;
@@ -324,6 +487,73 @@ extern "C" int mspr_flash_prefill(const void* q, const void* k, const void* v, i
   a.q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
   MSPR_REQUIRE((int64_t)a.q_blocks * n_kv_heads * batch < ((int64_t)1 << 31), "flash_prefill: grid too large");
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == MSPR_BF16) return prefill_launch<MSPR_BF16>(a, st);
-  return prefill_launch<MSPR_F16>(a, st);
+  if (dtype == MSPR_BF16) return prefill_launch<MSPR_BF16, false, MSPR_F32>(a, st);
+  return prefill_launch<MSPR_F16, false, MSPR_F32>(a, st);
+}
+
+extern "C" size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_kv_heads, int q_len, int64_t past_len) {
+  if (batch < 1 || n_kv_heads < 1 || q_len < 1 || past_len < 0) return 0;
+  const int64_t tail_rows = past_len % kTile + q_len;
+  return (size_t)batch * n_kv_heads * tail_rows * kRowBytes * 2 + 256;
+}
+
+extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, const void* pk_scales,
+                                       const void* pk_biases, const void* pv_wq, const void* pv_scales,
+                                       const void* pv_biases, int sb_dtype, const void* self_k, const void* self_v,
+                                       int self_dtype, int batch, int n_q_heads, int n_kv_heads, int head_dim,
+                                       int q_len, int64_t past_len, float scale, int group_size, int bits, void* out,
+                                       void* workspace, size_t workspace_bytes, void* stream) {
+  MSPR_REQUIRE(group_size == 64 && bits == 8, "sdpa_fa_prefill_q8: only group_size=64, bits=8 is supported");
+  MSPR_REQUIRE(queries && self_k && self_v && out, "sdpa_fa_prefill_q8: null pointer");
+  MSPR_REQUIRE(past_len == 0 || (pk_wq && pk_scales && pk_biases && pv_wq && pv_scales && pv_biases),
+               "sdpa_fa_prefill_q8: null pointer");
+  MSPR_REQUIRE(sb_dtype >= MSPR_F32 && sb_dtype <= MSPR_BF16 && self_dtype >= MSPR_F32 && self_dtype <= MSPR_BF16,
+               "sdpa_fa_prefill_q8: scales/biases and the self chunk must be f32, f16 or bf16");
+  MSPR_REQUIRE(head_dim == kD, "sdpa_fa_prefill_q8: head_dim must be 256");
+  MSPR_REQUIRE(batch >= 1 && n_kv_heads >= 1 && n_q_heads >= n_kv_heads && n_q_heads % n_kv_heads == 0,
+               "sdpa_fa_prefill_q8: bad head counts");
+  const int rep = n_q_heads / n_kv_heads;
+  MSPR_REQUIRE(rep == 1 || rep == 2 || rep == 4 || rep == 8,
+               "sdpa_fa_prefill_q8: query heads per KV head must be 1, 2, 4 or 8");
+  MSPR_REQUIRE(q_len >= 1 && past_len >= 0 && past_len + q_len < ((int64_t)1 << 31),
+               "sdpa_fa_prefill_q8: need q_len >= 1 and past_len >= 0");
+  MSPR_REQUIRE(mspr_aligned(queries, 16) && mspr_aligned(out, 16) && mspr_aligned(pk_wq, 16) && mspr_aligned(pv_wq, 16),
+               "sdpa_fa_prefill_q8: pointers must be 16-byte aligned");
+  const size_t need = mspr_sdpa_fa_prefill_q8_workspace_bytes(batch, n_kv_heads, q_len, past_len);
+  MSPR_REQUIRE(workspace && workspace_bytes >= need && mspr_aligned(workspace, 16),
+               "sdpa_fa_prefill_q8: workspace of %zu bytes (16-byte aligned) needed, %zu given", need, workspace_bytes);
+  PrefillArgs a = {};
+  const int tail_rows = (int)(past_len % kTile) + q_len;
+  uint16_t* tail_k = reinterpret_cast<uint16_t*>(workspace);
+  uint16_t* tail_v = tail_k + (size_t)batch * n_kv_heads * tail_rows * kD;
+  a.q = queries;
+  a.k = tail_k;
+  a.v = tail_v;
+  a.out = out;
+  a.batch = batch;
+  a.n_q_heads = n_q_heads;
+  a.n_kv_heads = n_kv_heads;
+  a.q_len = q_len;
+  a.past_len = past_len;
+  a.kv_rows = tail_rows;
+  a.scale_log2 = (float)((double)scale * 1.4426950408889634);
+  a.rep_shift = rep == 1 ? 0 : rep == 2 ? 1 : rep == 4 ? 2 : 3;
+  const int rows_per_wg = 32 * (8 / rep);
+  a.q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
+  a.q8_tiles = (int)(past_len / kTile);
+  a.pk_wq = pk_wq;
+  a.pk_s = pk_scales;
+  a.pk_b = pk_biases;
+  a.pv_wq = pv_wq;
+  a.pv_s = pv_scales;
+  a.pv_b = pv_biases;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 tgrid((unsigned)tail_rows, (unsigned)n_kv_heads, (unsigned)batch);
+  if (sb_dtype == MSPR_F32) prefill_q8_tail_kernel<MSPR_F32><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows);
+  else if (sb_dtype == MSPR_F16) prefill_q8_tail_kernel<MSPR_F16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows);
+  else prefill_q8_tail_kernel<MSPR_BF16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows);
+  MSPR_CHECK_LAUNCH("sdpa_fa_prefill_q8 (tail rows)");
+  if (sb_dtype == MSPR_F32) return prefill_launch<MSPR_F16, true, MSPR_F32>(a, st);
+  if (sb_dtype == MSPR_F16) return prefill_launch<MSPR_F16, true, MSPR_F16>(a, st);
+  return prefill_launch<MSPR_F16, true, MSPR_BF16>(a, st);
 }

@@ -125,6 +125,57 @@ def sdpa_decode_q8_0(queries, k_codes, k_scales, v_codes, v_scales, scale, *, wo
     return out
 
 
+def sdpa_fa_prefill_q8(queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, pv_biases, self_k, self_v, scale, *,
+                       group_size: int = 64, bits: int = 8, workspace=None, **_tuning):
+    """Causal flash prefill over a quantised prefix plus the dense chunk (reference call site full_attention.py:372).
+
+    Args:
+        queries: float32 ``[B, Hq, L, 256]`` (already rotated).
+        pk_* / pv_*: the affine 8-bit prefix of ``P`` tokens as read from the cache *before* the chunk
+            was appended (``P`` may be 0).
+        self_k, self_v: ``[B, Hkv, L, 256]`` float32/float16/bfloat16, the chunk's own keys and values
+            after the 8-bit round trip.
+        scale: softmax scale.
+
+    Returns:
+        float32 ``[B, Hq, L, 256]``; row ``i`` attends all prefix keys and chunk keys ``[0, i]``.
+    """
+    if group_size != 64 or bits != 8:
+        raise ValueError("sdpa_fa_prefill_q8 supports group_size=64, bits=8 only")
+    if queries.ndim != 4 or int(queries.shape[3]) != _HEAD_DIM:
+        raise ValueError("queries must be [B, Hq, L, 256]")
+    if queries.dtype != torch.float32:
+        raise ValueError("queries must be float32")
+    B, Hq, L = int(queries.shape[0]), int(queries.shape[1]), int(queries.shape[2])
+    _check_q8_triplet("past key", pk_wq, pk_scales, pk_biases, B)
+    P = int(pk_wq.shape[2])
+    _check_q8_triplet("past value", pv_wq, pv_scales, pv_biases, B, P)
+    Hkv = int(pk_wq.shape[1])
+    if pk_scales.dtype != pv_scales.dtype:
+        raise ValueError("key and value scales must share a dtype")
+    if self_k.ndim != 4 or tuple(self_k.shape) != (B, Hkv, L, _HEAD_DIM) or tuple(self_v.shape) != tuple(self_k.shape):
+        raise ValueError("self_k and self_v must be [B, Hkv, L, 256] with the chunk length of queries")
+    if self_k.dtype != self_v.dtype or self_k.dtype not in _lib.DTYPE_CODE:
+        raise ValueError("self_k and self_v must share a float32/float16/bfloat16 dtype")
+    if Hq % Hkv != 0 or Hq // Hkv not in (1, 2, 4, 8):
+        raise ValueError("query heads per KV head must be 1, 2, 4 or 8")
+    if L < 1:
+        raise ValueError("the chunk must hold at least one token")
+    _lib.require_device(queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, pv_biases, self_k, self_v)
+    q, kw, ks, kb, vw, vs, vb, sk, sv = [
+        t.contiguous() for t in (queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, pv_biases, self_k, self_v)]
+    out = torch.empty_like(q)
+    if workspace is None:
+        nbytes = int(_lib.lib().mspr_sdpa_fa_prefill_q8_workspace_bytes(B, Hkv, L, P))
+        workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=q.device)
+    _lib.check(_lib.lib().mspr_sdpa_fa_prefill_q8(
+        _lib.ptr(q), _lib.ptr(kw), _lib.ptr(ks), _lib.ptr(kb), _lib.ptr(vw), _lib.ptr(vs), _lib.ptr(vb),
+        _lib.DTYPE_CODE[ks.dtype], _lib.ptr(sk), _lib.ptr(sv), _lib.DTYPE_CODE[sk.dtype], B, Hq, Hkv, _HEAD_DIM, L, P,
+        float(scale), 64, 8, _lib.ptr(out), _lib.ptr(workspace), workspace.numel() * workspace.element_size(),
+        _lib.stream_ptr()), "sdpa_fa_prefill_q8")
+    return out
+
+
 def flash_prefill(queries, keys, values, scale, *, past_len: int):
     """Causal chunked-prefill GQA attention over a dense 16-bit cache that already holds the chunk.
 
