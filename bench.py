@@ -34,6 +34,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel at batch 16 (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
+# the same counters' reading for a 1 GiB elementwise kernel; profiles/bench_sparse_decode_layer_hbm_counters.txt)
+SPLIT_TRAFFIC_BYTES_B16 = 75_350_000
 
 # workload constants (BASELINE configs 4 and 5)
 N_IDX_HEADS, IDX_DIM, N_KEYS, TOPK = 64, 128, 32768, 2048
@@ -104,6 +107,84 @@ def cpu_baseline(seconds_budget: float = 15.0):
     }
 
 
+def cpu_config1():
+    """BASELINE config 1 (dense GQA decode, 8 q heads / 1 KV head, D=128, 4096 keys, fp16) on the host: the NumPy
+    restatement of softmax attention, warm-up 3, 20 repeats."""
+    from oracle import qwen
+
+    rng = np.random.default_rng(0)
+    q = rng.standard_normal((1, 8, 1, 128)).astype(np.float16)
+    k = rng.standard_normal((1, 1, 4096, 128)).astype(np.float16)
+    v = rng.standard_normal((1, 1, 4096, 128)).astype(np.float16)
+    for _ in range(3):
+        qwen.gqa_decode_attention(q, k, v, 128 ** -0.5)
+    t0 = time.perf_counter()
+    for _ in range(20):
+        qwen.gqa_decode_attention(q, k, v, 128 ** -0.5).astype(np.float16)
+    return {"us": round((time.perf_counter() - t0) / 20 * 1e6, 1), "kind": "port", "cores": min(16, os.cpu_count() or 1),
+            "workload": "dense GQA decode, 8q/1kv heads, D=128, 4096 fp16 keys (BASELINE config 1), NumPy float64"}
+
+
+def bench_prefill(dev, gen, reps=5):
+    """BASELINE config 2: 4096-token bf16 chunk over a 32768-token prefix, 16 q / 2 KV heads, D=256."""
+    from moespresso_amd import _lib
+    from moespresso_amd.runtime.qwen import kquant
+
+    L, past = 4096, 32768
+    q = (0.5 * torch.randn((1, 16, L, 256), device=dev, generator=gen)).to(torch.bfloat16)
+    k = (0.5 * torch.randn((1, 2, past + L, 256), device=dev, generator=gen)).to(torch.bfloat16)
+    v = (0.5 * torch.randn((1, 2, past + L, 256), device=dev, generator=gen)).to(torch.bfloat16)
+    for _ in range(2):
+        kquant.flash_prefill(q, k, v, 256 ** -0.5, past_len=past)
+    torch.cuda.synchronize()
+    _lib.profile_enable("flash_prefill")
+    for _ in range(reps):
+        kquant.flash_prefill(q, k, v, 256 ** -0.5, past_len=past)
+    torch.cuda.synchronize()
+    ms = float(np.mean(_lib.profile_collect("flash_prefill")))
+    _lib.profile_enable()
+    flops = 4.0 * 256 * 16 * (L * past + L * (L + 1) / 2)
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"ms": round(ms, 4), "TFLOPs": round(tf, 1), "peak_TFLOPs": 2500.0, "frac": round(tf / 2500.0, 4),
+            "tokens_per_s": round(L / (ms * 1e-3), 1), "bound": "mfma",
+            "workload": "causal prefill, 4096 new x 32768 prefix, 16q/2kv heads, D=256, bf16 (BASELINE config 2)"}
+
+
+def bench_q8_decode(dev, gen, reps=40):
+    """BASELINE config 3: GQA decode over a Q8_0 cache of 37000 tokens, batch 1 and 8."""
+    from moespresso_amd import _lib
+    from moespresso_amd.runtime.qwen import kquant
+
+    N, out = 37000, {}
+    for B in (1, 8):
+        sets = []
+        for _ in range(4):  # 4 x 322 MB at batch 8: beyond the 256 MB Infinity Cache
+            kc = torch.randint(-127, 128, (B, 2, N, 256), device=dev, dtype=torch.int8, generator=gen)
+            vc = torch.randint(-127, 128, (B, 2, N, 256), device=dev, dtype=torch.int8, generator=gen)
+            ks = (torch.rand((B, 2, N, 8), device=dev, generator=gen) * 0.03).half()
+            vs = (torch.rand((B, 2, N, 8), device=dev, generator=gen) * 0.03).half()
+            q = torch.randn((B, 16, 256), device=dev, generator=gen).to(torch.bfloat16)
+            sets.append((q, kc, ks, vc, vs))
+        ws = _lib.q8_decode_workspace(B, 2, N, dev)
+        for s_ in sets:
+            kquant.sdpa_decode_q8_0(*s_, 256 ** -0.5, workspace=ws)
+        torch.cuda.synchronize()
+        _lib.profile_enable("q8_decode", "q8_merge")
+        for i in range(reps):
+            kquant.sdpa_decode_q8_0(*sets[i % 4], 256 ** -0.5, workspace=ws)
+        torch.cuda.synchronize()
+        split = float(np.mean(_lib.profile_collect("q8_decode"))) * 1e3
+        merge = float(np.mean(_lib.profile_collect("q8_merge"))) * 1e3
+        _lib.profile_enable()
+        nbytes = B * (N * 2 * 2 * (256 + 16) + 16 * 256 * 4)
+        out[f"B{B}"] = {"split_us": round(split, 2), "merge_us": round(merge, 2),
+                        "GBps": round(nbytes / ((split + merge) * 1e-6) / 1e9, 1),
+                        "frac_of_8TBps": round(nbytes / ((split + merge) * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+        del sets
+    out["workload"] = "GQA decode, 16q/2kv heads, D=256, 37000-token int8+f16/32 cache (BASELINE config 3)"
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -112,6 +193,9 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--sets", type=int, default=8, help="distinct buffer sets rotated through (cold caches)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one elementwise kernel that reads 1 GiB and writes 1 GiB (scale for HBM counters)")
+    ap.add_argument("--headline-only", action="store_true", help="skip the per-config extras")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every box has one MI355X); rerun with --gpus 1",
@@ -184,16 +268,54 @@ def main() -> int:
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": None,
+        "traffic": SPLIT_TRAFFIC_BYTES_B16 if B == 16 else None,
         "algorithmic_bytes_per_launch": MLA_BYTES_PER_SEQ * B,
         "kernel_us": round(split_us, 2),
     }
+    # the same kernels at the smaller batches of the configuration (first sequences of the same buffers)
+    by_batch = {}
+    for bsub in (1, 4):
+        if bsub >= B:
+            continue
+        ws_b = _lib.sparse_attention_workspace(bsub, N_HEADS, TOPK + WINDOW, dev)
+        subsets = [{k_: v_[:bsub] for k_, v_ in s_.items()} for s_ in sets]
+
+        def step_b(s_):
+            sc = isk.indexer_scores_fp8(s_["qi"], s_["keys"], s_["kscale"], s_["w"])
+            se = isk.topk_select(sc, TOPK)
+            return iak.sparse_mla_decode(s_["q"], s_["kv"], se, scale=scale, window_start=N_TOKENS - WINDOW,
+                                         window_rows=WINDOW, row_mul=4, row_add=3, workspace=ws_b)
+
+        for s_ in subsets:
+            step_b(s_)
+        torch.cuda.synchronize()
+        _lib.profile_enable(*names)
+        for i in range(min(K, 64)):
+            step_b(subsets[i % R])
+        torch.cuda.synchronize()
+        by_batch[f"B{bsub}"] = {n_: round(float(np.mean(_lib.profile_collect(n_))) * 1e3, 2) for n_ in names}
+        _lib.profile_enable()
+    by_batch[f"B{B}"] = {k: round(v, 2) for k, v in kernel_us.items()}
+    del sets, graphs, outs
+    torch.cuda.empty_cache()
+
     extras = {
         "kernel_us": {k: round(v, 2) for k, v in kernel_us.items()},
+        "kernel_us_by_batch": by_batch,
+        "prefill": None if args.headline_only else bench_prefill(dev, gen),
+        "q8_decode": None if args.headline_only else bench_q8_decode(dev, gen),
+        "cpu_config1": None if args.no_cpu_baseline else cpu_config1(),
         "indexer_fp8_GBps": round(IDX_BYTES_PER_SEQ * B / (kernel_us["indexer_fp8"] * 1e-6) / 1e9, 1),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
         "buffer_sets": R,
     }
+    if args.calibration_copy:
+        src = torch.ones(1 << 28, device=dev, dtype=torch.float32)
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
+
     line = {
         "metric": "sparse decode attn us/layer @128K ctx (indexer score + top-2048 + indexed MLA decode)",
         "value": round(ms_per_step * 1e3, 2),
