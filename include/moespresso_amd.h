@@ -99,6 +99,22 @@ int mspr_indexer_scores_fp8(const void* q, const void* keys, const float* key_sc
                             const float* weights, int batch, int n_heads, int64_t n_rows,
                             float* scores, void* stream);
 
+/* Prefill-side QAT of query rows: the Hadamard of mspr_indexer_qat_rows with the group scale
+ * 2^ceil(log2(amax/6)) and ties in the lattice search going to the even lattice index.
+ * Replaces indexer_q_qat_live, indexed_attention_kernel.py:1989 (kernel :1125-1202).
+ * q/out: f32 [n_rows,128] (the [batch,n_heads,tokens,128] tensor, contiguous). */
+int mspr_indexer_q_qat_live(const float* q, int64_t n_rows, float* out, void* stream);
+
+/* Prefill-side indexer scores over a chunk:
+ *   scores[b,t,c] = sum_h max(q[b,h,t] . comp[b,c], 0) * weights[b,t,h], -inf where c >= (pos0+t+1)/ratio
+ * with both operands staged as float16 (ratio 0 = whole pool visible).
+ * Replaces indexer_scores_tiled_live, indexed_attention_kernel.py:1888 (kernel :1028-1122).
+ * q: [batch,n_heads,n_tokens,128], index_comp: [batch,n_comp,128], both of dtype (f32|f16);
+ * weights: f32 [batch,n_tokens,n_heads]; scores: f32 [batch,n_tokens,n_comp]. n_heads <= 64. */
+int mspr_indexer_scores_tiled_live(const void* q, const float* weights, const void* index_comp, int dtype,
+                                   int batch, int n_heads, int n_tokens, int64_t n_comp, int64_t pos0,
+                                   int ratio, float* scores, void* stream);
+
 /* ------------------------------------------------------------------ DS4 sparse attention */
 
 /* Scratch bytes for the three gathered-attention entry points below. */
@@ -115,6 +131,26 @@ int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, const void*
                                         int top_k, const float* sinks, int64_t pos0, int window,
                                         int ratio, int raw_start, float* out, void* workspace,
                                         size_t workspace_bytes, void* stream);
+
+/* Indexed mixed attention for every token of a prefill chunk: token t (position pos0+t) attends
+ * the ring rows for positions [max(first_raw, pos0+t+1-window), pos0+t], where the newest ring
+ * row holds position pos0+n_tokens-1, then its own topk ids under the rules of the decode form
+ * with visible = min((pos0+t+1)/ratio, n_comp).
+ * Replaces indexed_mixed_attention_prefill (:2030), indexed_mixed_attention_prefill_live_f16
+ * (:1571), _live_f32 (:1679) and banded_prefill_attention_live (:1782) of
+ * indexed_attention_kernel.py; the three layouts differ only in strides.
+ * q: element (b,t,head,:) at b*q_batch_stride + t*q_token_stride + head*q_head_stride (elements),
+ * 512 contiguous values of q_dtype (f32 rounded to half on load, or f16); raw_kv: f16
+ * [batch,raw_cap,512]; comp_kv: f16 [batch,n_comp,512]; topk: int32 [batch,n_tokens,top_k]
+ * (top_k may be 0); sinks: f32 [n_heads]; out: f32 with the strides of q.
+ * Workspace: mspr_sparse_attention_workspace_bytes(batch*n_tokens, n_heads, min(window or raw_cap, raw_cap) + top_k). */
+int mspr_indexed_mixed_attention_prefill(const void* q, int q_dtype, int batch, int n_heads, int n_tokens,
+                                         int64_t q_batch_stride, int64_t q_head_stride,
+                                         int64_t q_token_stride, const void* raw_kv, int raw_cap,
+                                         const void* comp_kv, int64_t n_comp, const int32_t* topk, int top_k,
+                                         const float* sinks, int64_t pos0, int window, int ratio,
+                                         int raw_start, float* out, void* workspace, size_t workspace_bytes,
+                                         void* stream);
 
 /* Decode SDPA of the fused island: rope(q), softmax over the window (row substituted at
  * params[1]) + pooled[sel] + per-head sink, float16 output, inverse rope.

@@ -36,6 +36,13 @@ SIGNATURES = {
                 c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "mspr_indexer_scores_fp8": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p, c_void_p]),
+    "mspr_indexer_q_qat_live": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
+    "mspr_indexer_scores_tiled_live": (
+        c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int64, c_int64, c_int, c_void_p,
+                c_void_p]),
+    "mspr_indexed_mixed_attention_prefill": (
+        c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64,
+                c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_sparse_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),
     "mspr_indexed_mixed_attention_decode": (
         c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int64,

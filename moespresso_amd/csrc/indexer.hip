@@ -31,6 +31,9 @@ __device__ __forceinline__ float mx_floor_max(float x, float fl) { return isnan(
 // [4l, 4l+3]. Follows the reference's float32 operation sequence: radix-2 butterflies in
 // increasing stride order, scale, per-32 group amax, power-of-two scale, clip, first-wins
 // nearest lattice value.
+// LIVE selects the prefill-side variant (indexed_attention_kernel.py:1125-1202 of the reference):
+// scale 2^ceil(log2(amax/6)) taken exactly, ties to the even lattice index.
+template <bool LIVE = false>
 __device__ __forceinline__ f32x4_t qat128(f32x4_t v, int lane32) {
   float a0 = v.x + v.y, a1 = v.x - v.y, a2 = v.z + v.w, a3 = v.z - v.w;
   f32x4_t x = {a0 + a2, a1 + a3, a0 - a2, a1 - a3};
@@ -54,7 +57,21 @@ __device__ __forceinline__ f32x4_t qat128(f32x4_t v, int lane32) {
     amax = (isnan(amax) || isnan(o)) ? __builtin_nanf("") : fmaxf(amax, o);
   }
   amax = mx_floor_max(amax, kAmaxFloor);
-  float scale = pow2_group_scale(amax, 6.0f);
+  float scale;
+  if constexpr (LIVE) {
+    const float r = amax / 6.0f;
+    const uint32_t u = __float_as_uint(r);
+    if (isnan(r) || isinf(r)) {
+      scale = r;
+    } else {
+      int e;
+      const float m = frexpf(r, &e);  // r = m * 2^e, m in [0.5, 1)
+      scale = ldexpf(1.0f, m == 0.5f ? e - 1 : e);
+    }
+    (void)u;
+  } else {
+    scale = pow2_group_scale(amax, 6.0f);
+  }
   const float lattice[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
   f32x4_t out;
 #pragma unroll
@@ -65,12 +82,14 @@ __device__ __forceinline__ f32x4_t qat128(f32x4_t v, int lane32) {
     float absn = fabsf(n);
     float best = fabsf(absn - lattice[0]);
     float dq = lattice[0];
+    bool best_odd = false;
 #pragma unroll
     for (int k = 1; k < 8; k++) {
       float d = fabsf(absn - lattice[k]);
-      if (d < best) {
+      if (d < best || (LIVE && d == best && (k & 1) == 0 && best_odd)) {
         best = d;
         dq = lattice[k];
+        best_odd = (k & 1) != 0;
       }
     }
     dq = n < 0.0f ? -dq : dq;
@@ -98,7 +117,7 @@ __device__ __forceinline__ f32x4_t load_row4(const void* base, int64_t row, int 
 }
 
 // ------------------------------------------------------------------ QAT rows
-template <int DT>
+template <int DT, bool LIVE = false>
 __global__ __launch_bounds__(256) void qat_rows_kernel(const void* __restrict__ x, int64_t n_rows,
                                                        float* __restrict__ out) {
   int lane32 = threadIdx.x & 31;
@@ -106,7 +125,7 @@ __global__ __launch_bounds__(256) void qat_rows_kernel(const void* __restrict__ 
   // rows past the end recompute the last row so every lane stays active for the shuffles
   int64_t src = row < n_rows ? row : n_rows - 1;
   f32x4_t v = load_row4<DT>(x, src, lane32);
-  f32x4_t y = qat128(v, lane32);
+  f32x4_t y = qat128<LIVE>(v, lane32);
   if (row < n_rows) reinterpret_cast<f32x4_t*>(out + row * 128)[lane32] = y;
 }
 
@@ -353,6 +372,16 @@ extern "C" int mspr_indexer_qat_rows(const void* x, int x_dtype, int64_t n_rows,
   else if (x_dtype == MSPR_F16) qat_rows_kernel<MSPR_F16><<<grid, block, 0, st>>>(x, n_rows, out);
   else qat_rows_kernel<MSPR_BF16><<<grid, block, 0, st>>>(x, n_rows, out);
   MSPR_CHECK_LAUNCH("indexer_qat_rows");
+  return MSPR_OK;
+}
+
+extern "C" int mspr_indexer_q_qat_live(const float* q, int64_t n_rows, float* out, void* stream) {
+  MSPR_REQUIRE(q && out, "indexer_q_qat_live: null pointer");
+  MSPR_REQUIRE(n_rows > 0, "indexer_q_qat_live: expects at least one row");
+  MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(out, 16), "indexer_q_qat_live: pointers must be 16-byte aligned");
+  dim3 grid((unsigned)((n_rows + 7) / 8)), block(256);
+  qat_rows_kernel<MSPR_F32, true><<<grid, block, 0, (hipStream_t)stream>>>(q, n_rows, out);
+  MSPR_CHECK_LAUNCH("indexer_q_qat_live");
   return MSPR_OK;
 }
 

@@ -43,9 +43,15 @@ struct SparseAttnArgs {
   // query
   const void* q;
   int q_dtype;
-  int64_t q_batch_stride;  // elements
+  int64_t q_batch_stride;  // elements; q of (b, t, head) at b*q_batch_stride + t*q_token_stride + head*q_head_stride
+  int64_t q_head_stride;
+  int64_t q_token_stride;
   int n_heads;
-  int batch;
+  int batch;               // sequences = batch entries x tokens
+  int n_tokens;            // query tokens per batch entry; they share the window and pool tensors
+  // prefill form: window range and visible pool prefix follow from the token's position pos0 + t
+  int prefill;
+  uint32_t pos0, window, ratio;
   // window segment
   const void* win;
   int64_t win_batch_stride;
@@ -84,6 +90,8 @@ struct SparseAttnArgs {
   // output
   void* out;
   int out_dtype;
+  int64_t out_batch_stride, out_head_stride, out_token_stride;  // elements
+  int direct;  // one key range per sequence: the split kernel normalises and stores, no partials
   long long* trace;  // debug builds only
 };
 
@@ -159,6 +167,46 @@ __device__ __forceinline__ void async_load_16(uint64_t src, uint32_t lds_base) {
 }
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Normalised output values of four consecutive columns -> output tensor, in the output element type
+// (the fused-decode form applies the inverse partial rope on the float16 values at float16 op rounding).
+template <int ODT>
+__device__ __forceinline__ void emit_output(const SparseAttnArgs& a, const float (&r)[4], int64_t ooff, int dim0) {
+  if constexpr (ODT == MSPR_F32) {
+    *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.out) + ooff) = f32x4_t{r[0], r[1], r[2], r[3]};
+  } else if constexpr (ODT == MSPR_BF16) {
+    u32x2_t w2 = {(uint32_t)f32_to_bf16_bits(r[0]) | ((uint32_t)f32_to_bf16_bits(r[1]) << 16),
+                  (uint32_t)f32_to_bf16_bits(r[2]) | ((uint32_t)f32_to_bf16_bits(r[3]) << 16)};
+    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + ooff) = w2;
+  } else {
+    float h[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) h[j] = f16_bits_to_f32(f32_to_f16_bits(r[j]));
+    if (a.rope && dim0 >= kDV - 64) {
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        int p = (dim0 - (kDV - 64)) / 2 + j;
+        float theta = (float)a.params[0] * a.inv_freq[p];
+        float cs = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
+        float sn = f16_bits_to_f32(f32_to_f16_bits(-(float)sin((double)theta)));
+        float x0 = h[2 * j], x1 = h[2 * j + 1];
+        float m0 = f16_bits_to_f32(f32_to_f16_bits(x0 * cs)), m1 = f16_bits_to_f32(f32_to_f16_bits(x1 * sn));
+        float m2 = f16_bits_to_f32(f32_to_f16_bits(x0 * sn)), m3 = f16_bits_to_f32(f32_to_f16_bits(x1 * cs));
+        h[2 * j] = f16_bits_to_f32(f32_to_f16_bits(m0 - m1));
+        h[2 * j + 1] = f16_bits_to_f32(f32_to_f16_bits(m2 + m3));
+      }
+    }
+    u32x2_t w2 = {(uint32_t)f32_to_f16_bits(h[0]) | ((uint32_t)f32_to_f16_bits(h[1]) << 16),
+                  (uint32_t)f32_to_f16_bits(h[2]) | ((uint32_t)f32_to_f16_bits(h[3]) << 16)};
+    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + ooff) = w2;
+  }
+}
+
+__device__ __forceinline__ float load_sink_log2(const SparseAttnArgs& a, int head) {
+  if (!a.sinks) return -__builtin_inff();
+  return (a.sinks_dtype == MSPR_F16 ? f16_bits_to_f32(reinterpret_cast<const uint16_t*>(a.sinks)[head])
+                                    : reinterpret_cast<const float*>(a.sinks)[head]) * 1.4426950408889634f;
+}
+
 template <int DK>
 struct Geometry {
   static constexpr int kSlots = DK / 8 + 1;        // 16-byte slots per LDS row; the last one is padding, so
@@ -211,9 +259,29 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   const int sp = work % a.n_splits;
   const int bh = work / a.n_splits;
   const int hb = bh % a.n_hblk;
-  const int b = bh / a.n_hblk;
+  const int seq = bh / a.n_hblk;
+  const int b = seq / a.n_tokens;
+  const int t = seq - b * a.n_tokens;
 
-  const int n_keys = a.n_win + a.n_idx;
+  // window rows and visible pool prefix of this sequence; the prefill form derives them from the
+  // token's position in the unsigned 32-bit arithmetic of the reference kernel
+  int seq_n_win = a.n_win, seq_win_first = a.win_first;
+  int64_t seq_visible = a.visible;
+  if (a.prefill) {
+    const uint32_t qpos = a.pos0 + (uint32_t)t, n_raw = (uint32_t)a.raw_cap;
+    const uint32_t last_pos = a.pos0 + (uint32_t)a.n_tokens - 1u;
+    const uint32_t first_raw_pos = last_pos + 1u - n_raw;
+    const uint32_t window_first = (a.window != 0u && qpos + 1u > a.window) ? qpos + 1u - a.window : 0u;
+    const uint32_t first = first_raw_pos > window_first ? first_raw_pos : window_first;
+    const uint32_t last = qpos < last_pos ? qpos : last_pos;
+    seq_n_win = first <= last ? (int)(last - first + 1u) : 0;
+    if (seq_n_win > a.n_win) seq_n_win = a.n_win;  // the host sized the slot space for n_win window rows
+    seq_win_first = first <= last ? (int)(first - first_raw_pos) : 0;
+    const int64_t vis = a.ratio == 0u ? a.n_pool : (int64_t)((qpos + 1u) / a.ratio);
+    seq_visible = vis < a.n_pool ? vis : a.n_pool;
+  }
+
+  const int n_keys = seq_n_win + a.n_idx;
   const int slot0 = sp * a.slots_per_split;
   int slot1 = slot0 + a.slots_per_split;
   if (slot1 > n_keys) slot1 = n_keys;
@@ -221,13 +289,14 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 
   const uint16_t* win_b = reinterpret_cast<const uint16_t*>(a.win) + (int64_t)b * a.win_batch_stride;
   const uint16_t* pool_b = reinterpret_cast<const uint16_t*>(a.pool) + (int64_t)b * a.pool_batch_stride;
-  const int32_t* idx_b = a.idx + (int64_t)b * a.idx_batch_stride;
+  const int32_t* idx_b = a.idx + (int64_t)seq * a.idx_batch_stride;
 
   MSPR_STAMP(0);
   // ---- query operand loads go out first: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7]
   const int head = hb * 64 + hg * 32 + n;
   const bool q_live = head < a.n_heads;
-  const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)(q_live ? head : 0) * DK + dh * G::kHalf + 8 * g;
+  const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)t * a.q_token_stride +
+                       (int64_t)(q_live ? head : 0) * a.q_head_stride + dh * G::kHalf + 8 * g;
   u32x4_t qf[G::kSteps];
   f32x4_t qraw32[QDT == MSPR_F32 ? G::kSteps : 1][2];
   if constexpr (QDT == MSPR_F32) {
@@ -256,15 +325,15 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     int first = a.n_idx;
     for (int i = tid; i < a.n_idx; i += kThreads) {
       int id = idx_b[i];
-      if (id >= 0 && (int64_t)id >= a.visible && i < first) first = i;
+      if (id >= 0 && (int64_t)id >= seq_visible && i < first) first = i;
     }
     if (first < a.n_idx) atomicMin(stop_shared, first);
     __syncthreads();
     stop_pos = *stop_shared;
   }
   const int subst_slot = a.subst_from_params ? a.params[1] : a.subst_slot;
-  const int id_base = slot0 > a.n_win ? slot0 - a.n_win : 0;           // first gathered index of the range
-  const int id_count = slot1 > a.n_win ? slot1 - a.n_win - id_base : 0;  // <= kMaxIds by construction
+  const int id_base = slot0 > seq_n_win ? slot0 - seq_n_win : 0;           // first gathered index of the range
+  const int id_count = slot1 > seq_n_win ? slot1 - seq_n_win - id_base : 0;  // <= kMaxIds by construction
   for (int i = tid; i < id_count; i += kThreads) ids[i] = id_base + i < stop_pos ? idx_b[id_base + i] : -1;
 
   // ---- static part of this thread's tile loads: LDS slot P = tid + 256 j holds (row P / kSlots, chunk P % kSlots)
@@ -283,16 +352,16 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     uint64_t ptr = zero_row;
     bool valid = false;
     if (slot < slot1) {
-      if (slot < a.n_win) {
+      if (slot < seq_n_win) {
         valid = true;
         if (slot == subst_slot) {
           ptr = reinterpret_cast<uint64_t>(a.subst_row);
         } else {
-          uint32_t r = ((uint32_t)a.raw_start + (uint32_t)a.win_first + (uint32_t)slot) % (uint32_t)a.raw_cap;
+          uint32_t r = ((uint32_t)a.raw_start + (uint32_t)seq_win_first + (uint32_t)slot) % (uint32_t)a.raw_cap;
           ptr = reinterpret_cast<uint64_t>(win_b + (int64_t)r * DK);
         }
       } else {
-        const int id = ids[slot - a.n_win - id_base];
+        const int id = ids[slot - seq_n_win - id_base];
         if (id >= 0) {
           const int64_t r = (int64_t)id * a.row_mul + a.row_add;
           if (r >= 0 && r < a.n_pool) {
@@ -510,9 +579,34 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   }
 
   MSPR_STAMP(4 + 6 * n_tiles);
-  // ---- partial results: registers go out in their native order (coalesced), stats per head
   float l_tot = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
-  const int64_t part = ((int64_t)(b * a.n_hblk + hb) * a.n_splits + sp);
+  if (a.direct) {
+    // ---- the only key range of this sequence: sink, normalise, store
+    const float sink = q_live ? load_sink_log2(a, head) : -__builtin_inff();
+    const float m_all = fmaxf(m_run, sink);
+    const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
+    const float w = fast_exp2(m_run - m_safe);
+    const float l = l_tot * w + fast_exp2(sink - m_safe);
+    const float f = l == 0.0f ? 0.0f : w / l;
+    if (q_live) {
+      const int64_t obase = (int64_t)b * a.out_batch_stride + (int64_t)t * a.out_token_stride +
+                            (int64_t)head * a.out_head_stride;
+#pragma unroll
+      for (int mt = 0; mt < 8; mt++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const float r[4] = {oacc[mt][4 * c] * f, oacc[mt][4 * c + 1] * f, oacc[mt][4 * c + 2] * f,
+                              oacc[mt][4 * c + 3] * f};
+          const int dim0 = dh * 256 + 32 * mt + 8 * c + 4 * g;
+          if (a.out_dtype == MSPR_F32) emit_output<MSPR_F32>(a, r, obase + dim0, dim0);
+          else if (a.out_dtype == MSPR_BF16) emit_output<MSPR_BF16>(a, r, obase + dim0, dim0);
+          else emit_output<MSPR_F16>(a, r, obase + dim0, dim0);
+        }
+    }
+    return;
+  }
+  // ---- partial results: registers go out in their native order (coalesced), stats per head
+  const int64_t part = ((int64_t)(seq * a.n_hblk + hb) * a.n_splits + sp);
   float* wo = a.ws_o + (part * 4 + wave) * (int64_t)(8 * 16 * 64);
 #pragma unroll
   for (int mt = 0; mt < 8; mt++)
@@ -538,19 +632,16 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   const int wave = (blockIdx.x >> 3) & 3;
   const int bh = blockIdx.x >> 5;
   const int hb = bh % a.n_hblk;
-  const int b = bh / a.n_hblk;
+  const int seq = bh / a.n_hblk;
+  const int b = seq / a.n_tokens;
+  const int t = seq - b * a.n_tokens;
   const int hg = wave >> 1, dh = wave & 1;
   const int n = lane & 31, g = lane >> 5;
   const int head = hb * 64 + hg * 32 + n;
   if (head >= a.n_heads) return;
 
-  const float kLog2e = 1.4426950408889634f;
-  float sink = -__builtin_inff();
-  if (a.sinks) {
-    sink = (a.sinks_dtype == MSPR_F16 ? f16_bits_to_f32(reinterpret_cast<const uint16_t*>(a.sinks)[head])
-                                      : reinterpret_cast<const float*>(a.sinks)[head]) * kLog2e;
-  }
-  const int64_t part0 = (int64_t)(b * a.n_hblk + hb) * a.n_splits;
+  const float sink = load_sink_log2(a, head);
+  const int64_t part0 = (int64_t)(seq * a.n_hblk + hb) * a.n_splits;
   const float* ml0 = a.ws_ml + (part0 * 64 + hg * 32 + n) * 2;
   const float* wo0 = a.ws_o + (part0 * 4 + wave) * (int64_t)(8 * 16 * 64) + ((mt * 4 + c) * 64 + lane) * 4;
   constexpr int kChunk = 8;
@@ -586,36 +677,9 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   const float inv = l == 0.0f ? 0.0f : 1.0f / l;
   float r[4] = {o.x * inv, o.y * inv, o.z * inv, o.w * inv};
   const int dim0 = dh * 256 + 32 * mt + 8 * c + 4 * g;
-  const int64_t ooff = ((int64_t)b * a.n_heads + head) * kDV + dim0;
-  if constexpr (ODT == MSPR_F32) {
-    *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.out) + ooff) = f32x4_t{r[0], r[1], r[2], r[3]};
-  } else if constexpr (ODT == MSPR_BF16) {
-    u32x2_t w2 = {(uint32_t)f32_to_bf16_bits(r[0]) | ((uint32_t)f32_to_bf16_bits(r[1]) << 16),
-                  (uint32_t)f32_to_bf16_bits(r[2]) | ((uint32_t)f32_to_bf16_bits(r[3]) << 16)};
-    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + ooff) = w2;
-  } else {
-    float h[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) h[j] = f16_bits_to_f32(f32_to_f16_bits(r[j]));
-    if (a.rope && dim0 >= kDV - 64) {
-      // inverse partial rope on the float16 output at float16 op rounding
-#pragma unroll
-      for (int j = 0; j < 2; j++) {
-        int p = (dim0 - (kDV - 64)) / 2 + j;
-        float theta = (float)a.params[0] * a.inv_freq[p];
-        float cs = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
-        float sn = f16_bits_to_f32(f32_to_f16_bits(-(float)sin((double)theta)));
-        float x0 = h[2 * j], x1 = h[2 * j + 1];
-        float m0 = f16_bits_to_f32(f32_to_f16_bits(x0 * cs)), m1 = f16_bits_to_f32(f32_to_f16_bits(x1 * sn));
-        float m2 = f16_bits_to_f32(f32_to_f16_bits(x0 * sn)), m3 = f16_bits_to_f32(f32_to_f16_bits(x1 * cs));
-        h[2 * j] = f16_bits_to_f32(f32_to_f16_bits(m0 - m1));
-        h[2 * j + 1] = f16_bits_to_f32(f32_to_f16_bits(m2 + m3));
-      }
-    }
-    u32x2_t w2 = {(uint32_t)f32_to_f16_bits(h[0]) | ((uint32_t)f32_to_f16_bits(h[1]) << 16),
-                  (uint32_t)f32_to_f16_bits(h[2]) | ((uint32_t)f32_to_f16_bits(h[3]) << 16)};
-    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + ooff) = w2;
-  }
+  const int64_t ooff = (int64_t)b * a.out_batch_stride + (int64_t)t * a.out_token_stride +
+                       (int64_t)head * a.out_head_stride + dim0;
+  emit_output<ODT>(a, r, ooff, dim0);
 }
 
 int choose_splits(int batch_hblk, int n_keys) {
@@ -635,6 +699,7 @@ int choose_splits(int batch_hblk, int n_keys) {
 size_t workspace_bytes(int batch, int n_heads, int64_t n_keys) {
   int n_hblk = (n_heads + 63) / 64;
   int splits = choose_splits(batch * n_hblk, (int)n_keys);
+  if (splits == 1) return 256;  // one key range per sequence: stored directly, no partials
   size_t parts = (size_t)batch * n_hblk * splits;
   return parts * (4 * 8 * 16 * 64 * sizeof(float)) + parts * 64 * 2 * sizeof(float) + 256;
 }
@@ -664,6 +729,12 @@ int launch_split(const SparseAttnArgs& a, hipStream_t st) {
 int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* workspace, size_t workspace_bytes_given,
                          hipStream_t st) {
   const int n_keys = a.n_win + a.n_idx;
+  if (a.n_tokens < 1) a.n_tokens = 1;
+  if (a.q_head_stride == 0) a.q_head_stride = k_dim;
+  if (a.out_head_stride == 0) {
+    a.out_head_stride = kDV;
+    a.out_batch_stride = (int64_t)a.n_heads * kDV;
+  }
   a.n_hblk = (a.n_heads + 63) / 64;
   a.n_splits = choose_splits(a.batch * a.n_hblk, n_keys);
   int sps = (n_keys + a.n_splits - 1) / a.n_splits;
@@ -672,6 +743,7 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   if (sps > 1024) sps = 1024;
   a.slots_per_split = sps;
   MSPR_REQUIRE((int64_t)sps * a.n_splits >= n_keys, "sparse attention: too many key slots (%d)", n_keys);
+  a.direct = a.n_splits == 1;
   size_t need = workspace_bytes(a.batch, a.n_heads, n_keys);
   MSPR_REQUIRE(workspace && workspace_bytes_given >= need, "sparse attention: workspace of %zu bytes needed, %zu given",
                need, workspace_bytes_given);
@@ -689,7 +761,7 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   else if (kv_dtype == MSPR_BF16 && k_dim == 512) rc = launch_split<MSPR_BF16, 512, kQSame, false>(a, st);
   else if (kv_dtype == MSPR_F16 && k_dim == 576) rc = launch_split<MSPR_F16, 576, kQSame, false>(a, st);
   else rc = launch_split<MSPR_F16, 512, kQSame, false>(a, st);
-  if (rc != MSPR_OK) return rc;
+  if (rc != MSPR_OK || a.direct) return rc;
   dim3 grid((unsigned)(a.batch * a.n_hblk * 32)), block(256);
   {
     MsprProfScope prof(MSPR_K_SPARSE_MERGE, st);
@@ -854,4 +926,74 @@ extern "C" int mspr_sparse_mla_decode(const void* q, const void* kv, const int32
   a.out = out;
   a.out_dtype = dtype;
   return run_sparse_attention(a, dtype, k_dim, workspace, workspace_bytes_given, (hipStream_t)stream);
+}
+
+extern "C" int mspr_indexed_mixed_attention_prefill(const void* q, int q_dtype, int batch, int n_heads, int n_tokens,
+                                                    int64_t q_batch_stride, int64_t q_head_stride,
+                                                    int64_t q_token_stride, const void* raw_kv, int raw_cap,
+                                                    const void* comp_kv, int64_t n_comp, const int32_t* topk,
+                                                    int top_k, const float* sinks, int64_t pos0, int window,
+                                                    int ratio, int raw_start, float* out, void* workspace,
+                                                    size_t workspace_bytes_given, void* stream) {
+  const char* what = "indexed_mixed_attention_prefill";
+  MSPR_REQUIRE(q && raw_kv && comp_kv && sinks && out, "%s: null pointer", what);
+  MSPR_REQUIRE(top_k == 0 || topk, "%s: null topk", what);
+  MSPR_REQUIRE(q_dtype == MSPR_F32 || q_dtype == MSPR_F16, "%s: q must be float16 or float32", what);
+  MSPR_REQUIRE(batch >= 1 && n_tokens >= 1 && n_heads >= 1, "%s: q must contain at least one batch, token and head",
+               what);
+  MSPR_REQUIRE((int64_t)batch * n_tokens < ((int64_t)1 << 24), "%s: too many tokens", what);
+  MSPR_REQUIRE(raw_cap >= 1, "%s: raw_kv must contain at least one row", what);
+  MSPR_REQUIRE(raw_start >= 0 && raw_start < raw_cap, "%s: raw_start must be inside raw_kv", what);
+  MSPR_REQUIRE(n_comp >= 1 && top_k >= 0 && window >= 0 && ratio >= 0 && pos0 >= 0 &&
+                   pos0 + n_tokens < ((int64_t)1 << 31),
+               "%s: bad size argument", what);
+  MSPR_REQUIRE(q_head_stride >= 512 && q_token_stride >= 0 && q_batch_stride >= 0 && q_head_stride % 8 == 0 &&
+                   q_token_stride % 8 == 0 && q_batch_stride % 8 == 0,
+               "%s: q strides must be multiples of 8 elements", what);
+  MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(raw_kv, 16) && mspr_aligned(comp_kv, 16) && mspr_aligned(out, 16),
+               "%s: pointers must be 16-byte aligned", what);
+  SparseAttnArgs a = {};
+  a.q = q;
+  a.q_dtype = q_dtype;
+  a.q_batch_stride = q_batch_stride;
+  a.q_head_stride = q_head_stride;
+  a.q_token_stride = q_token_stride;
+  a.n_heads = n_heads;
+  a.batch = batch * n_tokens;
+  a.n_tokens = n_tokens;
+  a.prefill = 1;
+  a.pos0 = (uint32_t)pos0;
+  a.window = (uint32_t)window;
+  a.ratio = (uint32_t)ratio;
+  a.win = raw_kv;
+  a.win_batch_stride = (int64_t)raw_cap * 512;
+  // slot space: at most min(window, raw_cap, tokens seen so far) ring rows per token
+  int64_t max_win = window != 0 && window < raw_cap ? window : raw_cap;
+  if (max_win > pos0 + n_tokens) max_win = pos0 + n_tokens;
+  a.n_win = (int)max_win;
+  a.win_first = 0;
+  a.raw_start = raw_start;
+  a.raw_cap = raw_cap;
+  a.subst_row = nullptr;
+  a.subst_slot = -1;
+  a.pool = comp_kv;
+  a.pool_batch_stride = n_comp * 512;
+  a.n_pool = n_comp;
+  a.idx = topk;
+  a.idx_batch_stride = top_k;
+  a.n_idx = top_k;
+  a.visible = n_comp;
+  a.check_stop = 1;
+  a.row_mul = 1;
+  a.row_add = 0;
+  a.sinks = sinks;
+  a.sinks_dtype = MSPR_F32;
+  a.scale_log2 = (float)(1.4426950408889634 / sqrt(512.0));
+  a.rope = 0;
+  a.out = out;
+  a.out_dtype = MSPR_F32;
+  a.out_batch_stride = q_batch_stride;
+  a.out_head_stride = q_head_stride;
+  a.out_token_stride = q_token_stride;
+  return run_sparse_attention(a, MSPR_F16, 512, workspace, workspace_bytes_given, (hipStream_t)stream);
 }

@@ -20,11 +20,49 @@ log-sum-exp in a second launch.
 
 from __future__ import annotations
 
+import os
+
 import torch
 
 from moespresso_amd import _lib
 
 _HEAD_DIM = 512
+
+# Prefill consumer engagement counts by the variant the reference would have dispatched
+# (reference :34-48). One HIP kernel serves all three; the names record the dispatch decision so
+# A/B harnesses that read the counters keep working.
+_CONSUMER_CALL_COUNTS = {"mma": 0, "v2": 0, "v1": 0}
+_SCORES_TILED_CALL_COUNTS = {"f16": 0, "f32": 0}
+
+
+def prefill_consumer_call_counts() -> dict[str, int]:
+    """Return prefill consumer engagement counts by kernel variant (reference :41)."""
+    return dict(_CONSUMER_CALL_COUNTS)
+
+
+def indexer_scores_call_counts() -> dict[str, int]:
+    """Return tiled score kernel engagement counts by operand dtype (reference :46)."""
+    return dict(_SCORES_TILED_CALL_COUNTS)
+
+
+def indexer_score_operands(q, index_comp):
+    """Return the tiled score kernel operand pair in float32 (reference :51)."""
+    return q.to(torch.float32), index_comp.to(torch.float32)
+
+
+def _prefill_live_v2_enabled() -> bool:
+    """Gate of the reference's 32-heads-per-threadgroup consumer, read per call (reference :1401)."""
+    return os.environ.get("MOESPRESSO_DSV4_R4_PREFILL_CONSUMER_V2", "1") != "0"
+
+
+def _prefill_live_mma_enabled() -> bool:
+    """Gate of the reference's matrix-unit consumer, read per call (reference :1431)."""
+    return os.environ.get("MOESPRESSO_DSV4_R4_PREFILL_CONSUMER_MMA", "1") != "0"
+
+
+def _indexer_q_qat_v2_enabled() -> bool:
+    """Gate of the reference's shuffle-based QAT restructure (bit-identical math, reference :1982)."""
+    return os.environ.get("MOESPRESSO_DSV4_R4_PREFILL_QAT_V2", "1") != "0"
 
 
 def indexed_mixed_attention_decode(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
@@ -145,4 +183,266 @@ def sparse_mla_decode(q, kv, rows, *, scale: float, v_dim: int = 512, window_sta
         k_dim, 512, n_pool, n_rows, int(row_mul), int(row_add), win_start, window_rows, float(scale), _lib.ptr(out), _lib.ptr(ws),
         ws.numel() * 4, _lib.stream_ptr())
     _lib.check(rc, "sparse_mla_decode")
+    return out
+
+
+def _run_prefill(q, raw_kv, comp_kv, topk, sinks, *, batch, n_heads, n_tokens, strides, raw_cap, n_comp, pos0,
+                 window, ratio, raw_start):
+    """Launch the per-token indexed attention over tensors already validated; ``strides`` are the
+    (batch, head, token) element strides of ``q`` and of the float32 output."""
+    dev = _lib.require_device(q, raw_kv, comp_kv, topk, sinks)
+    top_k = int(topk.shape[-1])
+    out = torch.empty(q.shape, dtype=torch.float32, device=dev)
+    max_win = min(int(window), raw_cap) if int(window) != 0 else raw_cap
+    ws = _lib.sparse_attention_workspace(batch * n_tokens, n_heads, max_win + top_k, dev)
+    rc = _lib.lib().mspr_indexed_mixed_attention_prefill(
+        _lib.ptr(q), _lib.DTYPE_CODE[q.dtype], batch, n_heads, n_tokens, strides[0], strides[1], strides[2],
+        _lib.ptr(raw_kv), raw_cap, _lib.ptr(comp_kv), n_comp, _lib.ptr(topk) if top_k else None, top_k,
+        _lib.ptr(sinks), int(pos0), int(window), int(ratio), int(raw_start), _lib.ptr(out), _lib.ptr(ws),
+        ws.numel() * 4, _lib.stream_ptr())
+    _lib.check(rc, "indexed_mixed_attention_prefill")
+    return out
+
+
+def indexed_mixed_attention_prefill(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
+                                    ratio: int = 4, raw_start: int = 0):
+    """Batch-token indexed mixed attention, DS4-c layout (reference :2030).
+
+    Args:
+        q: float32 ``[tokens, n_heads, 512]`` query heads.
+        raw_kv: float16 ``[raw_cap, 512]`` local raw KV rows; the newest row holds position
+            ``pos0 + tokens - 1``.
+        comp_kv: float16 ``[n_comp, 512]`` compressed KV rows.
+        topk: int32 ``[tokens, top_k]`` selected compressed row ids.
+        sinks: float32 ``[n_heads]`` attention sink logits.
+
+    Returns:
+        float32 ``[tokens, n_heads, 512]``.
+    """
+    if q.ndim != 3 or raw_kv.ndim != 2 or comp_kv.ndim != 2:
+        raise ValueError("q must be rank-3 and raw_kv/comp_kv rank-2")
+    n_tokens, n_heads, head_dim = int(q.shape[0]), int(q.shape[1]), int(q.shape[2])
+    if n_tokens <= 0:
+        raise ValueError("q must contain at least one token")
+    if head_dim != _HEAD_DIM:
+        raise ValueError("DS4 indexed prefill probe currently requires head_dim=512")
+    if n_heads % 8 != 0:
+        raise ValueError("DS4 indexed prefill probe requires n_heads to be divisible by 8")
+    if int(raw_kv.shape[1]) != head_dim or int(comp_kv.shape[1]) != head_dim:
+        raise ValueError("raw_kv and comp_kv width must match q")
+    if topk.ndim != 2 or int(topk.shape[0]) != n_tokens:
+        raise ValueError("topk must have shape [tokens, top_k]")
+    if tuple(sinks.shape) != (n_heads,):
+        raise ValueError("sinks must have shape [n_heads]")
+    if q.dtype != torch.float32:
+        raise ValueError("q must be float32, matching DS4-c's q buffer contract")
+    if raw_kv.dtype != torch.float16 or comp_kv.dtype != torch.float16:
+        raise ValueError("raw_kv and comp_kv must be float16")
+    if topk.dtype != torch.int32:
+        topk = topk.to(torch.int32)
+    if sinks.dtype != torch.float32:
+        sinks = sinks.to(torch.float32)
+    raw_cap = int(raw_kv.shape[0])
+    if raw_cap <= 0:
+        raise ValueError("raw_kv must contain at least one row")
+    if not (0 <= int(raw_start) < raw_cap):
+        raise ValueError("raw_start must be inside raw_kv")
+    if int(comp_kv.shape[0]) <= 0:
+        raise ValueError("comp_kv must contain at least one row")
+    return _run_prefill(q.contiguous(), raw_kv.contiguous(), comp_kv.contiguous(), topk.contiguous(),
+                        sinks.contiguous(), batch=1, n_heads=n_heads, n_tokens=n_tokens,
+                        strides=(0, head_dim, n_heads * head_dim), raw_cap=raw_cap, n_comp=int(comp_kv.shape[0]),
+                        pos0=pos0, window=window, ratio=ratio, raw_start=raw_start)
+
+
+def _validate_live(q, raw_kv, comp_kv, topk, sinks, q_dtype, q_dtype_message, raw_start):
+    if q.ndim != 4 or raw_kv.ndim != 4 or comp_kv.ndim != 3:
+        raise ValueError("q/raw_kv/comp_kv must have live BHLD/B1LD/BPD layouts")
+    batch, n_heads, n_tokens, head_dim = (int(v) for v in q.shape)
+    if batch <= 0 or n_tokens <= 0:
+        raise ValueError("q must contain at least one batch and token")
+    if head_dim != _HEAD_DIM:
+        raise ValueError("DS4 indexed prefill probe currently requires head_dim=512")
+    if n_heads % 8 != 0:
+        raise ValueError("DS4 indexed prefill probe requires n_heads to be divisible by 8")
+    if int(raw_kv.shape[0]) != batch or int(comp_kv.shape[0]) != batch:
+        raise ValueError("raw_kv and comp_kv batch size must match q")
+    if int(raw_kv.shape[-1]) != head_dim or int(comp_kv.shape[-1]) != head_dim:
+        raise ValueError("raw_kv and comp_kv width must match q")
+    if topk.ndim != 3 or int(topk.shape[0]) != batch or int(topk.shape[1]) != n_tokens:
+        raise ValueError("topk must have shape [batch, tokens, top_k]")
+    if tuple(sinks.shape) != (n_heads,):
+        raise ValueError("sinks must have shape [n_heads]")
+    if q.dtype != q_dtype:
+        raise ValueError(q_dtype_message)
+    if raw_kv.dtype != torch.float16 or comp_kv.dtype != torch.float16:
+        raise ValueError("raw_kv and comp_kv must be float16")
+    raw_cap = int(raw_kv.shape[2])
+    if raw_cap <= 0:
+        raise ValueError("raw_kv must contain at least one row")
+    if not (0 <= int(raw_start) < raw_cap):
+        raise ValueError("raw_start must be inside raw_kv")
+    if int(raw_kv.shape[1]) != 1:
+        raise ValueError("q/raw_kv/comp_kv must have live BHLD/B1LD/BPD layouts")
+    if int(comp_kv.shape[1]) <= 0:
+        raise ValueError("comp_kv must contain at least one row")
+    return batch, n_heads, n_tokens, head_dim, raw_cap
+
+
+def _count_live_dispatch(n_heads: int) -> None:
+    # the reference's selection order (:1645-1676): mma for heads % 16 == 0, then v2 for % 32, else v1
+    if n_heads % 16 == 0 and _prefill_live_mma_enabled():
+        _CONSUMER_CALL_COUNTS["mma"] += 1
+    elif n_heads % 32 == 0 and _prefill_live_v2_enabled():
+        _CONSUMER_CALL_COUNTS["v2"] += 1
+    else:
+        _CONSUMER_CALL_COUNTS["v1"] += 1
+
+
+def _launch_live(q, raw_kv, comp_kv, topk, sinks, dims, *, pos0, window, ratio, raw_start):
+    batch, n_heads, n_tokens, head_dim, raw_cap = dims
+    if topk.dtype != torch.int32:
+        topk = topk.to(torch.int32)
+    if sinks.dtype != torch.float32:
+        sinks = sinks.to(torch.float32)
+    return _run_prefill(q.contiguous(), raw_kv.contiguous(), comp_kv.contiguous(), topk.contiguous(),
+                        sinks.contiguous(), batch=batch, n_heads=n_heads, n_tokens=n_tokens,
+                        strides=(n_heads * n_tokens * head_dim, n_tokens * head_dim, head_dim), raw_cap=raw_cap,
+                        n_comp=int(comp_kv.shape[1]), pos0=pos0, window=window, ratio=ratio, raw_start=raw_start)
+
+
+def indexed_mixed_attention_prefill_live_f16(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
+                                             ratio: int = 4, raw_start: int = 0):
+    """Indexed prefill attention on the live BHLD layout, float16 queries (reference :1571).
+
+    Args:
+        q: float16 ``[batch, n_heads, tokens, 512]``.
+        raw_kv: float16 ``[batch, 1, raw_cap, 512]``; comp_kv: float16 ``[batch, n_comp, 512]``.
+        topk: int32 ``[batch, tokens, top_k]``; sinks: float32 ``[n_heads]``.
+
+    Returns:
+        float32 ``[batch, n_heads, tokens, 512]``.
+    """
+    dims = _validate_live(q, raw_kv, comp_kv, topk, sinks, torch.float16,
+                          "live prefill probe requires q to be float16", raw_start)
+    _count_live_dispatch(dims[1])
+    return _launch_live(q, raw_kv, comp_kv, topk, sinks, dims, pos0=pos0, window=window, ratio=ratio,
+                        raw_start=raw_start)
+
+
+def indexed_mixed_attention_prefill_live_f32(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
+                                             ratio: int = 4, raw_start: int = 0):
+    """Indexed prefill attention on the live BHLD layout, float32 queries rounded to half on load
+    (reference :1679)."""
+    dims = _validate_live(q, raw_kv, comp_kv, topk, sinks, torch.float32,
+                          "live f32 prefill probe requires q to be float32", raw_start)
+    _count_live_dispatch(dims[1])
+    return _launch_live(q, raw_kv, comp_kv, topk, sinks, dims, pos0=pos0, window=window, ratio=ratio,
+                        raw_start=raw_start)
+
+
+def banded_prefill_attention_live(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int, ratio: int):
+    """Banded prefill attention: a ``window``-token local band plus every visible pooled row (reference :1782).
+
+    ``topk`` carries ascending pool row ids, so the visibility rule (id below ``(position+1)/ratio``)
+    reproduces the compressed-pool predicate. Zero-pool layers pass a one-row ``comp_kv`` with a
+    zero-width ``topk``.
+    """
+    if q.ndim != 4 or raw_kv.ndim != 4 or comp_kv.ndim != 3:
+        raise ValueError("q/raw_kv/comp_kv must have live BHLD/B1LD/BPD layouts")
+    batch, n_heads, n_tokens, head_dim = (int(v) for v in q.shape)
+    if batch <= 0 or n_tokens <= 0:
+        raise ValueError("q must contain at least one batch and token")
+    if head_dim != _HEAD_DIM:
+        raise ValueError("banded mma attention requires head_dim=512")
+    if n_heads % 16 != 0 or not _prefill_live_mma_enabled():
+        raise ValueError("banded mma attention requires the mma consumer")
+    if int(raw_kv.shape[0]) != batch or int(comp_kv.shape[0]) != batch:
+        raise ValueError("raw_kv and comp_kv batch size must match q")
+    if int(raw_kv.shape[-1]) != head_dim or int(comp_kv.shape[-1]) != head_dim:
+        raise ValueError("raw_kv and comp_kv width must match q")
+    if int(comp_kv.shape[1]) <= 0:
+        raise ValueError("comp_kv must contain at least one row")
+    if topk.ndim != 3 or int(topk.shape[0]) != batch or int(topk.shape[1]) != n_tokens:
+        raise ValueError("topk must have shape [batch, tokens, width]")
+    if q.dtype not in (torch.float16, torch.float32):
+        raise ValueError("banded mma attention requires q to be float16 or float32")
+    if raw_kv.dtype != torch.float16 or comp_kv.dtype != torch.float16:
+        raise ValueError("raw_kv and comp_kv must be float16")
+    if int(window) <= 0 or int(ratio) <= 0:
+        raise ValueError("banded mma attention requires positive window and ratio")
+    if tuple(sinks.shape) != (n_heads,):
+        raise ValueError("sinks must have shape [n_heads]")
+    raw_cap = int(raw_kv.shape[2])
+    if raw_cap <= 0:
+        raise ValueError("raw_kv must contain at least one row")
+    dims = (batch, n_heads, n_tokens, head_dim, raw_cap)
+    return _launch_live(q, raw_kv, comp_kv, topk, sinks, dims, pos0=pos0, window=window, ratio=ratio, raw_start=0)
+
+
+def indexer_scores_tiled_live(q, weights, index_comp, *, pos0: int, ratio: int = 4):
+    """Ratio-4 indexer scores over a prefill chunk (reference :1888).
+
+    Args:
+        q: float32 or float16 ``[batch, n_heads, tokens, 128]`` QAT indexer queries (staged as half).
+        weights: float32 ``[batch, tokens, n_heads]`` head weights including the DS4 scale factors.
+        index_comp: ``[batch, n_comp, 128]`` QAT compressed index rows, same dtype as ``q``.
+
+    Returns:
+        float32 ``[batch, tokens, n_comp]``, ``-inf`` where the row is not yet visible to the token.
+    """
+    if q.ndim != 4 or weights.ndim != 3 or index_comp.ndim != 3:
+        raise ValueError("q, weights, and index_comp must be BHLD/BLH/BPD")
+    batch, n_heads, n_tokens, head_dim = (int(v) for v in q.shape)
+    n_comp = int(index_comp.shape[1])
+    if batch <= 0 or n_tokens <= 0:
+        raise ValueError("q must contain at least one batch and token")
+    if head_dim != 128:
+        raise ValueError("DS4 indexer score probe requires head_dim=128")
+    if int(index_comp.shape[0]) != batch or int(index_comp.shape[2]) != head_dim:
+        raise ValueError("index_comp must have shape [batch, n_comp, 128]")
+    if tuple(weights.shape) != (batch, n_tokens, n_heads):
+        raise ValueError("weights must have shape [batch, tokens, n_heads]")
+    if weights.dtype != torch.float32:
+        raise ValueError("weights must be float32")
+    if q.dtype == torch.float16 or index_comp.dtype == torch.float16:
+        if q.dtype != torch.float16 or index_comp.dtype != torch.float16:
+            raise ValueError("half score operands require both q and index_comp as float16")
+        operand_form = "f16"
+    elif q.dtype == torch.float32 and index_comp.dtype == torch.float32:
+        operand_form = "f32"
+    else:
+        raise ValueError("q and index_comp must both be float32 or both be float16")
+    if n_comp <= 0:
+        raise ValueError("index_comp must contain at least one compressed row")
+    if n_heads > 64:
+        raise ValueError("DS4 indexer score probe supports between 1 and 64 heads")
+    dev = _lib.require_device(q, weights, index_comp)
+    _SCORES_TILED_CALL_COUNTS[operand_form] += 1
+    qc, wc, cc = q.contiguous(), weights.contiguous(), index_comp.contiguous()
+    scores = torch.empty((batch, n_tokens, n_comp), dtype=torch.float32, device=dev)
+    rc = _lib.lib().mspr_indexer_scores_tiled_live(
+        _lib.ptr(qc), _lib.ptr(wc), _lib.ptr(cc), _lib.DTYPE_CODE[qc.dtype], batch, n_heads, n_tokens, n_comp,
+        int(pos0), int(ratio), _lib.ptr(scores), _lib.stream_ptr())
+    _lib.check(rc, "indexer_scores_tiled_live")
+    return scores
+
+
+def indexer_q_qat_live(q):
+    """Hadamard-128 + FP4 QAT of live BHLD query rows, prefill-side rules (reference :1989)."""
+    if q.ndim != 4:
+        raise ValueError("q must have shape [batch, n_heads, tokens, 128]")
+    batch, n_heads, n_tokens, head_dim = (int(v) for v in q.shape)
+    if batch <= 0 or n_tokens <= 0:
+        raise ValueError("q must contain at least one batch and token")
+    if head_dim != 128:
+        raise ValueError("DS4 indexer QAT probe requires head_dim=128")
+    if q.dtype != torch.float32:
+        raise ValueError("q must be float32")
+    dev = _lib.require_device(q)
+    qc = q.contiguous()
+    out = torch.empty(qc.shape, dtype=torch.float32, device=dev)
+    rc = _lib.lib().mspr_indexer_q_qat_live(_lib.ptr(qc), batch * n_heads * n_tokens, _lib.ptr(out),
+                                            _lib.stream_ptr())
+    _lib.check(rc, "indexer_q_qat_live")
     return out

@@ -167,6 +167,73 @@ def indexer_qat(x: np.ndarray) -> np.ndarray:
     return indexer_fp4_act_roundtrip(hadamard128(x))
 
 
+def e2m1_nearest_prefer_even(absn: np.ndarray) -> np.ndarray:
+    """Nearest e2m1 lattice value of ``absn`` in [0, 6]; a tie goes to the even lattice index
+    (the scan of indexed_attention_kernel.py:1131-1141)."""
+    absn = np.asarray(absn, dtype=F32)
+    diff = np.abs(absn[..., None] - E2M1_LATTICE).astype(F32)
+    best = np.zeros(absn.shape, dtype=np.int64)
+    best_diff = diff[..., 0].copy()
+    for i in range(1, 8):
+        d = diff[..., i]
+        take = (d < best_diff) | ((d == best_diff) & (i % 2 == 0) & (best % 2 != 0))
+        best = np.where(take, i, best)
+        best_diff = np.where(take, d, best_diff)
+    return E2M1_LATTICE[best]
+
+
+def exp2_ceil_log2(x: np.ndarray) -> np.ndarray:
+    """``2 ** ceil(log2(x))`` for positive float32 ``x``, taken exactly from exponent and mantissa."""
+    m, e = np.frexp(np.asarray(x, dtype=F32))  # x = m * 2^e, m in [0.5, 1)
+    k = np.where(m == 0.5, e - 1, e)
+    return np.ldexp(F32(1.0), k).astype(F32)
+
+
+def indexer_q_qat_live(q: np.ndarray) -> np.ndarray:
+    """The prefill-side QAT kernel (indexed_attention_kernel.py:1125-1202, wrapper :1989).
+
+    Same Hadamard as a1, but the group scale is ``exp2(ceil(log2(amax/6)))`` and a tie in the
+    nearest-lattice search prefers the even lattice index (:1137-1141). Here ``ceil(log2(x))`` is
+    taken exactly from the float32 exponent/mantissa of ``amax/6`` (Metal's ``log2``/``exp2`` bits
+    within an ulp of a power of two are not knowable from the source: parity unpinned there; the
+    reference test holds this kernel to 1e-5 against a1 only, test_..._indexed_attention_kernel.py:266-285).
+    """
+    y = hadamard128(np.asarray(q, dtype=F32))
+    shape = y.shape
+    g = y.reshape(-1, shape[-1] // 32, 32)
+    with np.errstate(invalid="ignore", divide="ignore", over="ignore"):
+        amax = np.maximum(np.max(np.abs(g), axis=-1, keepdims=True), AMAX_FLOOR).astype(F32)
+        scale = exp2_ceil_log2((amax / F32(6.0)).astype(F32))
+        n = np.clip((g / scale).astype(F32), -6.0, 6.0)
+        dq = e2m1_nearest_prefer_even(np.abs(n))
+        dq = np.where(n < 0, -dq, dq).astype(F32)
+        out = (dq * scale).astype(F32)
+    return out.reshape(shape)
+
+
+def indexer_scores_tiled_live(q, weights, index_comp, *, pos0: int, ratio: int = 4) -> np.ndarray:
+    """Prefill-side indexer scores (indexed_attention_kernel.py:1028-1122, wrapper :1888).
+
+    ``scores[b,t,c] = sum_h max(q[b,h,t] . comp[b,c], 0) * w[b,t,h]`` with both operands staged as
+    float16, ``-inf`` where ``c >= (pos0+t+1)//ratio``. q ``[B,H,T,128]``, weights ``[B,T,H]``,
+    index_comp ``[B,P,128]`` -> float64 ``[B,T,P]``.
+    """
+    qh = round_f16(np.asarray(q, dtype=F32)).astype(np.float64)
+    ch = round_f16(np.asarray(index_comp, dtype=F32)).astype(np.float64)
+    w = np.asarray(weights, dtype=np.float64)
+    b, h, t, _ = qh.shape
+    p = ch.shape[1]
+    out = np.empty((b, t, p), dtype=np.float64)
+    for bi in range(b):
+        for ti in range(t):
+            raw = qh[bi, :, ti, :] @ ch[bi].T  # [H, P]
+            s = (np.maximum(raw, 0.0) * w[bi, ti][:, None]).sum(axis=0)
+            visible = p if ratio == 0 else min(p, (int(pos0) + ti + 1) // int(ratio))
+            s[visible:] = -np.inf
+            out[bi, ti] = s
+    return out
+
+
 # --------------------------------------------------------------------------
 # a10: E4M3FN KV round trip
 # --------------------------------------------------------------------------

@@ -416,3 +416,42 @@ def test_sparse_mla_and_fp8_indexer_closed_forms():
     k = torch.from_numpy(codes).view(torch.float8_e4m3fn).to(torch.float64).numpy() * ks[..., None]
     want = (np.maximum(np.einsum("bhd,bnd->bhn", qi.astype(np.float64), k), 0) * w[..., None]).sum(1)
     np.testing.assert_allclose(got, want, rtol=1e-12)
+
+
+def test_live_qat_matches_a1_off_midpoints_and_prefers_even_on_ties():
+    """indexed_attention_kernel.py:1137-1141: the live QAT differs from a1 only on exact midpoints
+    (even lattice index wins) and where exp(k ln2) is not exactly 2^k."""
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((64, 128)).astype(np.float32)
+    a1, live = ds4.indexer_qat(x), ds4.indexer_q_qat_live(x)
+    np.testing.assert_allclose(live, a1, rtol=1e-5, atol=1e-5)  # the reference test's own bar
+    mid = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], dtype=np.float32)  # the seven lattice midpoints
+    np.testing.assert_array_equal(ds4.e2m1_nearest_prefer_even(mid),
+                                  np.array([0.0, 1.0, 1.0, 2.0, 2.0, 4.0, 4.0], dtype=np.float32))
+    # off the midpoints it is plain nearest
+    np.testing.assert_array_equal(ds4.e2m1_nearest_prefer_even(np.array([0.2, 0.3, 1.6, 2.6, 5.1, 6.0], dtype=np.float32)),
+                                  np.array([0.0, 0.5, 1.5, 3.0, 6.0, 6.0], dtype=np.float32))
+    # a row whose groups have amax exactly 6 * 2^k after the Hadamard scale cannot be built exactly
+    # (the scale constant is not 2^-3.5), so the scale rule is pinned on its own: exact powers of two
+    x = np.array([1.0, 1.0000001, 0.5, 0.49999997, 2.0, 3.0, 2.0 ** -100, 1.5 * 2.0 ** -100], dtype=np.float32)
+    np.testing.assert_array_equal(ds4.exp2_ceil_log2(x),
+                                  np.array([1.0, 2.0, 0.5, 0.5, 2.0, 4.0, 2.0 ** -100, 2.0 ** -99], dtype=np.float32))
+
+
+def test_tiled_live_scores_closed_form_and_visibility():
+    rng = np.random.default_rng(12)
+    B, H, T, P = 2, 8, 5, 9
+    q = rng.standard_normal((B, H, T, 128)).astype(np.float32)
+    comp = rng.standard_normal((B, P, 128)).astype(np.float32)
+    w = rng.uniform(0, 1, (B, T, H)).astype(np.float32)
+    got = ds4.indexer_scores_tiled_live(q, w, comp, pos0=6, ratio=4)
+    qh, ch = q.astype(np.float16).astype(np.float64), comp.astype(np.float16).astype(np.float64)
+    for b in range(B):
+        for t in range(T):
+            visible = min(P, (6 + t + 1) // 4)
+            for c in range(P):
+                want = sum(max(float(qh[b, h, t] @ ch[b, c]), 0.0) * float(w[b, t, h]) for h in range(H))
+                if c < visible:
+                    assert abs(got[b, t, c] - want) < 1e-9
+                else:
+                    assert got[b, t, c] == -np.inf
