@@ -180,6 +180,17 @@ int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, c
 
 /* ------------------------------------------------------------------ Qwen/Ornith GQA attention, 8-bit KV */
 
+/* Affine 8-bit quantisation in groups of 64 over the last axis and its inverse: the cache write
+ * path in front of the two attention operators below.
+ * Stands in for mx.quantize / mx.dequantize (group_size=64, bits=8) as used by the quantised KV
+ * cache's update and by the self-chunk round trip, runtime/qwen/full_attention.py:352-369.
+ * x/out: [n_groups*64] of dtype (f32|f16|bf16); wq: uint32 [n_groups*16], four codes per word,
+ * lowest byte first; scales, biases: [n_groups] of dtype; value = code*scale + bias. */
+int mspr_affine_q8_quantize(const void* x, int dtype, int64_t n_groups, void* wq, void* scales,
+                            void* biases, int group_size, int bits, void* stream);
+int mspr_affine_q8_dequantize(const void* wq, const void* scales, const void* biases, int dtype,
+                              int64_t n_groups, void* out, int group_size, int bits, void* stream);
+
 /* Workspace bytes of the two Q8 decode entry points below. */
 size_t mspr_sdpa_decode_q8_workspace_bytes(int batch, int n_kv_heads, int64_t n_keys);
 

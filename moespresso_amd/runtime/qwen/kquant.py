@@ -21,6 +21,10 @@ from moespresso_amd import _lib
 
 _HEAD_DIM = 256
 
+# The decode kernel's range merge always spreads the 256 output columns over the merging waves;
+# the flag exists because callers probe for it (reference full_attention.py:146-157).
+HAS_SDPA_DECODE_Q8_DIMENSION_PARALLEL_MERGE = True
+
 
 def _check_q8_triplet(name, wq, scales, biases, batch, n_keys=None):
     if wq.ndim != 4 or scales.ndim != 4 or biases.ndim != 4:
@@ -38,6 +42,116 @@ def _check_q8_triplet(name, wq, scales, biases, batch, n_keys=None):
         raise ValueError(f"{name} codes, scales and biases disagree on [B, Hkv, N]")
     if n_keys is not None and int(wq.shape[2]) != n_keys:
         raise ValueError("keys and values disagree on the number of cached tokens")
+
+
+def quantize(x, group_size: int = 64, bits: int = 8):
+    """Affine 8-bit quantisation over the last axis (the role of ``mx.quantize`` on the cache write path).
+
+    Returns ``(wq uint32 [..., D/4], scales [..., D/64], biases [..., D/64])``; scales and biases in
+    the dtype of ``x``.
+    """
+    if group_size != 64 or bits != 8:
+        raise ValueError("quantize supports group_size=64, bits=8 only")
+    if x.dtype not in _lib.DTYPE_CODE:
+        raise ValueError("x must be float32, float16 or bfloat16")
+    if x.ndim < 1 or int(x.shape[-1]) % 64 != 0 or x.numel() == 0:
+        raise ValueError("the last axis must be a non-empty multiple of the group size 64")
+    dev = _lib.require_device(x)
+    xc = x.contiguous()
+    d = int(xc.shape[-1])
+    lead = tuple(xc.shape[:-1])
+    wq = torch.empty(lead + (d // 4,), dtype=torch.int32, device=dev).view(torch.uint32)
+    scales = torch.empty(lead + (d // 64,), dtype=xc.dtype, device=dev)
+    biases = torch.empty_like(scales)
+    _lib.check(_lib.lib().mspr_affine_q8_quantize(
+        _lib.ptr(xc), _lib.DTYPE_CODE[xc.dtype], xc.numel() // 64, _lib.ptr(wq), _lib.ptr(scales), _lib.ptr(biases),
+        64, 8, _lib.stream_ptr()), "quantize")
+    return wq, scales, biases
+
+
+def dequantize(wq, scales, biases, group_size: int = 64, bits: int = 8):
+    """``code * scale + bias`` in the dtype of ``scales`` (the role of ``mx.dequantize``)."""
+    if group_size != 64 or bits != 8:
+        raise ValueError("dequantize supports group_size=64, bits=8 only")
+    if scales.dtype not in _lib.DTYPE_CODE or biases.dtype != scales.dtype:
+        raise ValueError("scales and biases must share a float32/float16/bfloat16 dtype")
+    if wq.dtype not in (torch.uint32, torch.int32):
+        raise ValueError("codes must be uint32 words")
+    if tuple(scales.shape) != tuple(biases.shape) or tuple(wq.shape[:-1]) != tuple(scales.shape[:-1]) or \
+            int(wq.shape[-1]) != 16 * int(scales.shape[-1]) or wq.numel() == 0:
+        raise ValueError("codes, scales and biases disagree on the group layout")
+    dev = _lib.require_device(wq, scales, biases)
+    w, s, b = wq.contiguous(), scales.contiguous(), biases.contiguous()
+    out = torch.empty(tuple(w.shape[:-1]) + (int(w.shape[-1]) * 4,), dtype=s.dtype, device=dev)
+    _lib.check(_lib.lib().mspr_affine_q8_dequantize(
+        _lib.ptr(w), _lib.ptr(s), _lib.ptr(b), _lib.DTYPE_CODE[s.dtype], s.numel(), _lib.ptr(out), 64, 8,
+        _lib.stream_ptr()), "dequantize")
+    return out
+
+
+class QuantizedKVCache:
+    """Affine 8-bit KV cache with quantise-on-append (the role of mlx_lm's ``QuantizedKVCache`` in
+    runtime/qwen/full_attention.py:315,352-356).
+
+    ``keys`` / ``values`` are ``(wq, scales, biases)`` triplets over a capacity that grows in
+    ``step``-token blocks; ``offset`` tokens are valid. ``update_and_fetch`` quantises the new rows in
+    place behind the valid prefix and returns the triplets trimmed to the new length; ``state`` is the
+    same view without an update.
+    """
+
+    step = 256
+
+    def __init__(self, group_size: int = 64, bits: int = 8):
+        if group_size != 64 or bits != 8:
+            raise ValueError("QuantizedKVCache supports group_size=64, bits=8 only")
+        self.group_size = group_size
+        self.bits = bits
+        self.offset = 0
+        self.keys = None
+        self.values = None
+
+    def _grow(self, like, need: int):
+        B, H, _, D = (int(v) for v in like.shape)
+        cap = 0 if self.keys is None else int(self.keys[0].shape[2])
+        if need <= cap:
+            return
+        new_cap = (need + self.step - 1) // self.step * self.step
+
+        def alloc():
+            return (torch.zeros((B, H, new_cap, D // 4), dtype=torch.int32, device=like.device).view(torch.uint32),
+                    torch.zeros((B, H, new_cap, D // 64), dtype=like.dtype, device=like.device),
+                    torch.zeros((B, H, new_cap, D // 64), dtype=like.dtype, device=like.device))
+
+        new_k, new_v = alloc(), alloc()
+        if self.keys is not None and self.offset:
+            for old, new in zip(self.keys + self.values, new_k + new_v):
+                new[:, :, :self.offset].view(torch.int32 if new.dtype == torch.uint32 else new.dtype).copy_(
+                    old[:, :, :self.offset].view(torch.int32 if old.dtype == torch.uint32 else old.dtype))
+        self.keys, self.values = new_k, new_v
+
+    def _trimmed(self, triplet):
+        return tuple(t[:, :, :self.offset] for t in triplet)
+
+    @property
+    def state(self):
+        if self.keys is None:
+            return None, None
+        return self._trimmed(self.keys), self._trimmed(self.values)
+
+    def update_and_fetch(self, keys, values):
+        """Append ``keys``/``values`` ``[B, Hkv, L, D]`` and return the quantised cache up to the new length."""
+        if keys.ndim != 4 or tuple(keys.shape) != tuple(values.shape):
+            raise ValueError("keys and values must be [B, Hkv, L, D] of one shape")
+        L = int(keys.shape[2])
+        self._grow(keys, self.offset + L)
+        for src, dst in ((keys, self.keys), (values, self.values)):
+            wq, sc, bi = quantize(src)
+            lo, hi = self.offset, self.offset + L
+            dst[0][:, :, lo:hi].view(torch.int32).copy_(wq.view(torch.int32))
+            dst[1][:, :, lo:hi].copy_(sc)
+            dst[2][:, :, lo:hi].copy_(bi)
+        self.offset += L
+        return self._trimmed(self.keys), self._trimmed(self.values)
 
 
 def sdpa_decode_q8(queries, k_wq, k_scales, k_biases, v_wq, v_scales, v_biases, scale, *, group_size: int = 64,

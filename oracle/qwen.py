@@ -46,22 +46,23 @@ def affine_q8_quantize(x: np.ndarray, group_size: int = 64):
     """
     x = np.asarray(x, dtype=F32)
     d = x.shape[-1]
-    g = x.reshape(*x.shape[:-1], d // group_size, group_size).astype(np.float64)
+    g = x.reshape(*x.shape[:-1], d // group_size, group_size)
+    # float32 throughout, one rounding per operation (the order of the Metal kernel's statements)
     w_max = g.max(axis=-1, keepdims=True)
     w_min = g.min(axis=-1, keepdims=True)
-    mask = np.abs(w_min) > np.abs(w_max)
-    scales = np.maximum((w_max - w_min) / 255.0, 1e-7)
-    scales = np.where(mask, scales, -scales)
-    edge = np.where(mask, w_min, w_max)
-    q0 = np.rint(edge / scales)
-    scales = np.where(q0 != 0, edge / np.where(q0 != 0, q0, 1.0), scales)
-    biases = np.where(q0 == 0, 0.0, edge)
-    scales32 = scales.astype(F32)
-    biases32 = biases.astype(F32)
-    codes = np.clip(np.rint((g - biases32.astype(np.float64)) / scales32.astype(np.float64)), 0, 255)
-    codes = codes.astype(np.uint8).reshape(*x.shape[:-1], d)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        scales = np.maximum(((w_max - w_min).astype(F32) / F32(255.0)).astype(F32), F32(1e-7))
+        side = np.abs(w_min) > np.abs(w_max)
+        scales = np.where(side, scales, -scales).astype(F32)
+        edge = np.where(side, w_min, w_max).astype(F32)
+        q0 = np.rint((edge / scales).astype(F32))
+        at_zero = q0 == 0
+        scales = np.where(at_zero, scales, (edge / np.where(at_zero, F32(1.0), q0)).astype(F32)).astype(F32)
+        biases = np.where(at_zero, F32(0.0), edge).astype(F32)
+        codes = np.rint(((g - biases).astype(F32) / scales).astype(F32))
+    codes = np.clip(codes, 0, 255).astype(np.uint8).reshape(*x.shape[:-1], d)
     packed = np.ascontiguousarray(codes).view("<u4")
-    return packed, scales32[..., 0], biases32[..., 0]
+    return packed, scales[..., 0], biases[..., 0]
 
 
 def affine_q8_dequantize(packed: np.ndarray, scales: np.ndarray, biases: np.ndarray,

@@ -1,0 +1,154 @@
+"""GPU: affine 8-bit quantiser (bit-exact vs the oracle), the quantised KV cache, and the full-attention
+dispatch wrapper against a composed stand-in (dequantise + float32 softmax attention in torch)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import qwen
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    return torch.device("cuda:0")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_quantize_dequantize_bit_exact(dtype):
+    from moespresso_amd.runtime.qwen import kquant
+
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 2, 37, 256)).astype(np.float32)
+    x[0, 0, 0, :64] = 0.0                 # all-zero group: scale floor, bias 0
+    x[0, 0, 1, :64] = 1.25                # constant group
+    x[0, 0, 2, :64] = np.abs(x[0, 0, 2, :64])   # positive-only group
+    x[0, 0, 3, :64] = -np.abs(x[0, 0, 3, :64])  # negative-only group
+    xt = torch.from_numpy(x).to(dtype)
+    wq, sc, bi = kquant.quantize(xt.to(_dev()))
+    assert wq.dtype == torch.uint32 and sc.dtype == dtype and tuple(wq.shape) == (2, 2, 37, 64)
+    want_wq, want_sc, want_bi = qwen.affine_q8_quantize(xt.float().numpy())
+    np.testing.assert_array_equal(wq.view(torch.int32).cpu().numpy().view(np.uint32), want_wq)
+    np.testing.assert_array_equal(sc.float().cpu().numpy(), torch.from_numpy(want_sc).to(dtype).float().numpy())
+    np.testing.assert_array_equal(bi.float().cpu().numpy(), torch.from_numpy(want_bi).to(dtype).float().numpy())
+    back = kquant.dequantize(wq, sc, bi)
+    want_back = torch.from_numpy(qwen.affine_q8_dequantize(want_wq, sc.float().cpu().numpy(), bi.float().cpu().numpy()))
+    assert back.dtype == dtype
+    np.testing.assert_array_equal(back.float().cpu().numpy(), want_back.to(dtype).float().numpy())
+    # round-trip error is at most one step
+    step = np.abs(sc.float().cpu().numpy())[..., None]
+    err = np.abs(back.float().cpu().numpy() - xt.float().numpy()).reshape(2, 2, 37, 4, 64)
+    tol = 1.01 * step + (0.0 if dtype == torch.float32 else 0.02 * np.abs(xt.float().numpy()).reshape(2, 2, 37, 4, 64))
+    assert (err <= tol + 1e-6).all()
+
+
+def test_quantized_cache_appends_and_grows():
+    from moespresso_amd.runtime.qwen import kquant
+
+    g = torch.Generator().manual_seed(0)
+    cache = kquant.QuantizedKVCache(group_size=64, bits=8)
+    assert cache.state == (None, None) and cache.offset == 0
+    chunks = [torch.randn((1, 2, n, 256), generator=g) for n in (200, 100, 1, 300)]
+    for c in chunks:
+        k, v = cache.update_and_fetch(c.to(_dev()), (2 * c).to(_dev()))
+    total = sum(int(c.shape[2]) for c in chunks)
+    assert cache.offset == total and int(k[0].shape[2]) == total and int(cache.keys[0].shape[2]) % 256 == 0
+    full = torch.cat(chunks, dim=2)
+    want = qwen.affine_q8_quantize(full.numpy())
+    np.testing.assert_array_equal(k[0].view(torch.int32).cpu().numpy().view(np.uint32), want[0])
+    np.testing.assert_array_equal(k[1].cpu().numpy(), want[1])
+    sk, sv = cache.state
+    assert torch.equal(sk[0].view(torch.int32), k[0].view(torch.int32)) and int(sv[2].shape[2]) == total
+
+
+class _Block(torch.nn.Module):
+    """A small gated attention block with the attribute names the wrapper uses (random weights)."""
+
+    def __init__(self, hidden=64, heads=16, kv_heads=2, head_dim=256, seed=33):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.num_attention_heads, self.num_key_value_heads, self.scale = heads, kv_heads, head_dim ** -0.5
+        mk = lambda i, o: torch.nn.Parameter(torch.randn((o, i), generator=g) * i ** -0.5)
+        self.wq, self.wk = mk(hidden, 2 * heads * head_dim), mk(hidden, kv_heads * head_dim)
+        self.wv, self.wo = mk(hidden, kv_heads * head_dim), mk(heads * head_dim, hidden)
+        self.q_proj = lambda x: x @ self.wq.T
+        self.k_proj = lambda x: x @ self.wk.T
+        self.v_proj = lambda x: x @ self.wv.T
+        self.o_proj = lambda x: x @ self.wo.T
+        self.q_norm = self.k_norm = lambda x: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)
+        self.stock_calls = 0
+
+    def rope(self, x, offset=0):
+        # rotate the first 64 dims of each head by position-dependent angles
+        T = x.shape[2]
+        pos = torch.arange(offset, offset + T, device=x.device, dtype=torch.float32)
+        inv = 1.0 / (10000.0 ** (torch.arange(0, 32, device=x.device, dtype=torch.float32) / 32))
+        ang = pos[:, None] * inv[None, :]
+        c, s = ang.cos(), ang.sin()
+        a, b_, rest = x[..., :32], x[..., 32:64], x[..., 64:]
+        return torch.cat([a * c - b_ * s, a * s + b_ * c, rest], dim=-1)
+
+    def stock_attention(self, queries, keys, values, cache=None, scale=1.0, mask=None):
+        """Composed path: dequantise the cache, float32 softmax attention."""
+        from moespresso_amd.runtime.qwen import kquant
+
+        self.stock_calls += 1
+        if isinstance(keys, tuple):
+            keys, values = kquant.dequantize(*keys), kquant.dequantize(*values)
+        rep = queries.shape[1] // keys.shape[1]
+        k = keys.float().repeat_interleave(rep, dim=1)
+        v = values.float().repeat_interleave(rep, dim=1)
+        s = (queries.float() @ k.transpose(-1, -2)) * scale
+        if mask == "causal":
+            L, N = queries.shape[2], k.shape[2]
+            allowed = torch.arange(N, device=s.device)[None, :] <= (N - L + torch.arange(L, device=s.device))[:, None]
+            s = s.masked_fill(~allowed, float("-inf"))
+        return torch.softmax(s, dim=-1) @ v
+
+
+def _x(L, seed):
+    return torch.randn((1, L, 64), generator=torch.Generator().manual_seed(seed)).to(_dev())
+
+
+def test_wrapper_prefill_and_decode_match_composed_path(monkeypatch):
+    from moespresso_amd.runtime.qwen import full_attention as fa
+    from moespresso_amd.runtime.qwen import kquant
+
+    monkeypatch.setattr(fa, "_QWEN_PREFILL_FLASH_D256", True)
+    monkeypatch.setattr(fa, "_QWEN_DECODE_Q8_TILE16", True)
+    monkeypatch.setattr(fa, "_DECODE_Q8_TILE16_MIN_KEYS", 64)
+    stock = _Block().to(_dev())
+    wrapped = fa.FlashPrefillD256Attention(stock)
+    cache_w, cache_s = kquant.QuantizedKVCache(), kquant.QuantizedKVCache()
+
+    def stock_forward(x, mask, cache):  # the wrapper with every route declined
+        ref = fa.FlashPrefillD256Attention(stock)
+        monkeypatch.setattr(fa, "_QWEN_PREFILL_FLASH_D256", False)
+        monkeypatch.setattr(fa, "_QWEN_DECODE_Q8_TILE16", False)
+        try:
+            return ref(x, mask=mask, cache=cache)
+        finally:
+            monkeypatch.setattr(fa, "_QWEN_PREFILL_FLASH_D256", True)
+            monkeypatch.setattr(fa, "_QWEN_DECODE_Q8_TILE16", True)
+
+    with torch.no_grad():
+        # first chunk: empty cache -> declined (fallback_cache), both sides composed
+        out0_w = wrapped(_x(64, 40), mask="causal", cache=cache_w)
+        out0_s = stock_forward(_x(64, 40), "causal", cache_s)
+        assert wrapped.fallback_cache == 1 and wrapped.flash_calls == 0
+        assert torch.equal(out0_w, out0_s)
+        # second chunk: flash route
+        out1_w = wrapped(_x(48, 41), mask="causal", cache=cache_w)
+        out1_s = stock_forward(_x(48, 41), "causal", cache_s)
+        assert wrapped.flash_calls == 1 and cache_w.offset == cache_s.offset == 112
+        rel = ((out1_w - out1_s).norm() / out1_s.norm()).item()
+        assert rel < 2e-3, rel
+        # decode token: 8-bit decode route (112 + 1 >= 64 keys)
+        out2_w = wrapped(_x(1, 42), mask=None, cache=cache_w)
+        out2_s = stock_forward(_x(1, 42), None, cache_s)
+        assert wrapped.decode_calls == 1 and wrapped.decode_dimension_merge_calls == 1
+        rel = ((out2_w - out2_s).norm() / out2_s.norm()).item()
+        assert rel < 2e-3, rel
+        # no cache at all: declined and counted
+        wrapped(_x(8, 43), mask="causal", cache=None)
+        assert wrapped.fallback_no_cache == 1
