@@ -15,6 +15,22 @@
 #include "common.h"
 #include "profile.h"
 
+#ifdef MSPR_TOPK_TRACE
+// Debug build only: cycle stamps of the phases of workgroup 0.
+__device__ long long g_topk_trace[32];
+extern "C" int mspr_debug_topk_trace(long long* host_out) {
+  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_topk_trace), sizeof(long long) * 32);
+}
+#define TOPK_STAMP(i)                                                      \
+  do {                                                                     \
+    if (blockIdx.x == 0 && threadIdx.x == 0) g_topk_trace[i] = clock64(); \
+  } while (0)
+#else
+#define TOPK_STAMP(i) \
+  do {                \
+  } while (0)
+#endif
+
 namespace {
 
 constexpr int kThreads = 1024;
@@ -290,14 +306,256 @@ __global__ __launch_bounds__(kThreads) void topk_select_kernel(const float* __re
   }
 }
 
+// Every wave runs this on the same 256 totals and gets the same answer in every lane: the digit
+// where the count from the top first reaches `need`, the keys still needed inside it and its size.
+struct Pick {
+  uint32_t digit, need, live;
+};
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (no LDS round trips):
+// four shifts inside each row of 16 lanes, then the row totals are carried across rows.
+__device__ __forceinline__ uint32_t wave_prefix_sum(uint32_t x) {
+  int v = (int)x;
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+  return (uint32_t)v;
+}
+
+__device__ __forceinline__ Pick pick_bucket(const uint32_t* totals, uint32_t need, int lane) {
+  // lane l looks at digits 255-4l .. 252-4l, so a prefix sum over lanes counts keys from the top digit down
+  uint32_t t[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) t[j] = totals[255 - (4 * lane + j)];
+  const uint32_t lane_sum = t[0] + t[1] + t[2] + t[3];
+  const uint32_t incl = wave_prefix_sum(lane_sum);
+  int chosen = -1;
+  uint32_t chosen_need = 0u, chosen_cnt = 0u;
+  uint32_t run = incl - lane_sum;  // keys in higher digits
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    if (chosen < 0 && run < need && run + t[j] >= need) {
+      chosen = 255 - (4 * lane + j);
+      chosen_need = need - run;
+      chosen_cnt = t[j];
+    }
+    run += t[j];
+  }
+  const uint64_t any = __ballot(chosen >= 0);
+  Pick p;
+  if (any) {
+    const int src = (int)__builtin_ctzll(any);
+    p.digit = (uint32_t)__builtin_amdgcn_readlane(chosen, src);
+    p.need = (uint32_t)__builtin_amdgcn_readlane((int)chosen_need, src);
+    p.live = (uint32_t)__builtin_amdgcn_readlane((int)chosen_cnt, src);
+  } else {
+    // fewer keys than needed cannot happen for topk <= rows held; digit 0 would take the rest
+    const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)incl, 63);
+    const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)t[3], 63);
+    p.digit = 0u;
+    p.need = need - (total - d0);
+    p.live = d0;
+  }
+  return p;
+}
+
+// Rows of up to C*1024 scores: thread t owns the C consecutive rows [C t, C t + C) in registers.
+// With consecutive ownership the ordered emission needs no cross-lane work per row: a thread knows
+// the relative order of its own rows, so one packed block scan of the per-thread counts gives every
+// thread its output slots. Digit histograms over all keys use 256 bins x 64 copies (copy = lane, so
+// an LDS atomic never meets a bank conflict whatever the digit distribution); the thread that sums a
+// group of copies also zeroes it for the next pass. Select state lives in registers: every wave derives it
+// from the same totals, which saves the broadcast barriers.
+// Rows past n_rows are given key 0: they can only tie with the lowest possible key and lose every
+// tie to a real row (ties go to the lower index), so no pass needs a bounds check.
+template <int C>
+__global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __restrict__ scores_all,
+                                                                 int64_t score_stride, int n_rows, int topk,
+                                                                 int32_t* __restrict__ sel_all) {
+  // The staging area for the load (C*1024 keys) is reused for the histogram copies afterwards.
+  constexpr int kStageWords = C * kThreads > 256 * kCopies ? C * kThreads : 256 * kCopies;
+  __shared__ __attribute__((aligned(16))) uint32_t stage[kStageWords];
+  uint32_t* hist = stage;                   // [bin][copy]
+  __shared__ uint32_t totals[256];
+  __shared__ uint32_t small_hist[2][256];   // digits 2 and 3 on the compacted list
+  __shared__ uint32_t list[kListCap];
+  __shared__ uint32_t list_n;
+  __shared__ uint32_t wave_tot[kWaves];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const float* scores = scores_all + (int64_t)blockIdx.x * score_stride;
+  int32_t* sel = sel_all + (int64_t)blockIdx.x * topk;
+
+  TOPK_STAMP(0);
+  // Load with lane-contiguous 16-byte reads (a wave reads 1 KB at a time), then hand every thread its
+  // C consecutive rows through LDS. The 16-byte pieces of a thread's C/4-piece block are XOR-permuted
+  // by the thread index so that neither the writes nor the reads pile up on a few banks.
+  uint32_t kreg[C];
+  {
+    constexpr int kPieces = C / 4;  // 16-byte pieces per thread
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(scores) & 15u) == 0u && n_rows >= 4;  // uniform
+    // all vector loads first, unconditionally (a piece that crosses the end of the row re-reads the
+    // last whole piece and is patched element by element below)
+    f32x4_t v[kPieces];
+    const int last_whole = (n_rows - 4) & ~3;
+    if (vec_ok) {
+#pragma unroll
+      for (int k = 0; k < kPieces; k++) {
+        const int r = 4 * (k * kThreads + tid);
+        v[k] = *reinterpret_cast<const f32x4_t*>(scores + (r < last_whole ? r : last_whole));
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kPieces; k++) {
+      const int piece = k * kThreads + tid;  // global piece index: rows 4*piece .. 4*piece+3
+      const int r = 4 * piece;
+      u32x4_t keys;
+      if (vec_ok && r + 3 < n_rows) {
+        keys = u32x4_t{score_key(v[k].x), score_key(v[k].y), score_key(v[k].z), score_key(v[k].w)};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) keys[e] = r + e < n_rows ? score_key(scores[r + e]) : 0u;
+      }
+      const int owner = piece / kPieces, j = piece % kPieces;
+      *reinterpret_cast<u32x4_t*>(&stage[owner * C + 4 * (j ^ (owner & (kPieces - 1)))]) = keys;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kPieces; j++) {
+      const u32x4_t keys = *reinterpret_cast<const u32x4_t*>(&stage[tid * C + 4 * (j ^ (tid & (kPieces - 1)))]);
+#pragma unroll
+      for (int e = 0; e < 4; e++) kreg[4 * j + e] = keys[e];
+    }
+    __syncthreads();
+  }
+  {
+    u32x4_t* h4 = reinterpret_cast<u32x4_t*>(hist);
+    for (int i = tid; i < 256 * kCopies / 4; i += kThreads) h4[i] = u32x4_t{0u, 0u, 0u, 0u};
+    if (tid < 512) (&small_hist[0][0])[tid] = 0u;
+    if (tid == 0) list_n = 0u;
+  }
+  __syncthreads();
+  TOPK_STAMP(1);
+
+  uint32_t prefix = 0u, need = (uint32_t)topk, live = (uint32_t)(C * kThreads);
+
+  // one digit over every key of the thread
+  auto full_pass = [&](int pass) {
+    const uint32_t shift = 24u - 8u * pass;
+    const uint32_t mask_hi = pass == 0 ? 0u : (0xFFFFFFFFu << (shift + 8u));
+#pragma unroll
+    for (int i = 0; i < C; i++) {
+      const uint32_t key = kreg[i];
+      if (pass == 0 || (key & mask_hi) == prefix) atomicAdd(&hist[((key >> shift) & 0xFFu) * kCopies + lane], 1u);
+    }
+    TOPK_STAMP(2 + 3 * pass);
+    __syncthreads();
+    TOPK_STAMP(3 + 3 * pass);
+    // totals[bin] = sum over copies: four threads per bin, 16 copies each as four 16-byte reads
+    // (rotated so that 16 neighbouring lanes cover all 16 bank groups), zeroed behind the read
+    {
+      const int bin = tid >> 2, q = tid & 3;
+      uint32_t sum = 0u;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        u32x4_t* p = reinterpret_cast<u32x4_t*>(&hist[bin * kCopies + q * 16 + 4 * ((j + (tid >> 2)) & 3)]);
+        const u32x4_t v = *p;
+        *p = u32x4_t{0u, 0u, 0u, 0u};
+        sum += v.x + v.y + v.z + v.w;
+      }
+      sum += __shfl_xor(sum, 1, MSPR_WAVE);
+      sum += __shfl_xor(sum, 2, MSPR_WAVE);
+      if (q == 0) totals[bin] = sum;
+    }
+    __syncthreads();
+    const Pick p = pick_bucket(totals, need, lane);
+    prefix |= p.digit << shift;
+    need = p.need;
+    live = p.live;
+    TOPK_STAMP(4 + 3 * pass);
+  };
+
+  full_pass(0);
+  full_pass(1);
+
+  if (live <= (uint32_t)kListCap) {
+    // the keys that still match the 16-bit prefix are few: finish the select on a compacted list
+#pragma unroll
+    for (int i = 0; i < C; i++) {
+      const uint32_t key = kreg[i];
+      if ((key & 0xFFFF0000u) == prefix) list[atomicAdd(&list_n, 1u)] = key;
+    }
+    __syncthreads();
+    const uint32_t n_list = list_n;
+#pragma unroll
+    for (int pass = 2; pass < 4; pass++) {
+      const uint32_t shift = 24u - 8u * pass;
+      const uint32_t mask_hi = 0xFFFFFFFFu << (shift + 8u);
+      uint32_t* h = small_hist[pass - 2];
+      for (uint32_t i = tid; i < n_list; i += kThreads) {
+        const uint32_t key = list[i];
+        if ((key & mask_hi) == prefix) atomicAdd(&h[(key >> shift) & 0xFFu], 1u);
+      }
+      __syncthreads();
+      const Pick p = pick_bucket(h, need, lane);
+      prefix |= p.digit << shift;
+      need = p.need;
+      live = p.live;
+    }
+  } else {
+    full_pass(2);
+    full_pass(3);
+  }
+
+  const uint32_t threshold = prefix;
+  const uint32_t need_ties = need;
+  const uint32_t n_above = (uint32_t)topk - need_ties;
+  TOPK_STAMP(14);
+
+  // ---- ordered emission: per-thread masks, one packed block scan (above count low, tie count high)
+  uint32_t above_mask = 0u, tie_mask = 0u;
+#pragma unroll
+  for (int i = 0; i < C; i++) {
+    above_mask |= (kreg[i] > threshold ? 1u : 0u) << i;
+    tie_mask |= (kreg[i] == threshold ? 1u : 0u) << i;
+  }
+  const uint32_t mine = (uint32_t)__popc(above_mask) | ((uint32_t)__popc(tie_mask) << 16);
+  const uint32_t incl = wave_prefix_sum(mine);
+  if (lane == 63) wave_tot[wave] = incl;
+  TOPK_STAMP(15);
+  __syncthreads();
+  TOPK_STAMP(16);
+  uint32_t base = 0u;
+  for (int w = 0; w < wave; w++) base += wave_tot[w];
+  const uint32_t excl = base + incl - mine;
+  uint32_t slot_a = excl & 0xFFFFu;
+  uint32_t rank_t = excl >> 16;
+  const int row0 = C * tid;
+  while (above_mask) {
+    const int i = __builtin_ctz(above_mask);
+    above_mask &= above_mask - 1u;
+    sel[slot_a++] = row0 + i;
+  }
+  while (tie_mask && rank_t < need_ties) {
+    const int i = __builtin_ctz(tie_mask);
+    tie_mask &= tie_mask - 1u;
+    sel[n_above + rank_t++] = row0 + i;
+  }
+  TOPK_STAMP(17);
+}
+
 }  // namespace
 
 int mspr_launch_topk(const float* scores, int64_t score_stride, int batch, int64_t n_rows, int topk, int32_t* sel,
                      hipStream_t st) {
   dim3 grid((unsigned)batch), block(kThreads);
   MsprProfScope prof(MSPR_K_TOPK, st);
-  if (n_rows <= 8 * 1024) topk_select_kernel<8><<<grid, block, 0, st>>>(scores, score_stride, n_rows, topk, sel);
-  else if (n_rows <= 32 * 1024) topk_select_kernel<32><<<grid, block, 0, st>>>(scores, score_stride, n_rows, topk, sel);
+  if (n_rows <= 8 * 1024) topk_blocked_kernel<8><<<grid, block, 0, st>>>(scores, score_stride, (int)n_rows, topk, sel);
+  else if (n_rows <= 32 * 1024) topk_blocked_kernel<32><<<grid, block, 0, st>>>(scores, score_stride, (int)n_rows, topk, sel);
   else topk_select_kernel<0><<<grid, block, 0, st>>>(scores, score_stride, n_rows, topk, sel);
   MSPR_CHECK_LAUNCH("topk_select");
   return MSPR_OK;
