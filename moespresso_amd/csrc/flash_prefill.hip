@@ -21,9 +21,9 @@ constexpr int kRowBytes = kD * 2;
 constexpr int kTile = 32;                       // keys per tile
 constexpr int kTileBytes = kTile * kRowBytes;   // 16 KB, K and V each
 constexpr int kStageBytes = 2 * kTileBytes;
-constexpr int kBufs = 3;
+constexpr int kBufs = 4;
 constexpr int kThreads = 512;
-constexpr int kLdsBytes = kBufs * kStageBytes;  // 96 KB
+constexpr int kLdsBytes = kBufs * kStageBytes;  // 128 KB
 
 struct PrefillArgs {
   const void* q;   // [B, Hq, L, 256]
@@ -223,43 +223,48 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   const int my_last_key = past + q0 + 31;  // last key any query of this wave may see
   const int qpos = past + q0 + n;
 
-  auto compute_tile = [&](const unsigned char* st, int key0) {
+  // stage 1 of a tile: S^T = K . Q^T on the matrix cores
+  auto qk_tile = [&](const unsigned char* st, f32x16_t& sacc) {
     // S^T = K . Q^T
-    f32x16_t sacc = {0};
+    sacc = f32x16_t{0};
     {
-      constexpr int kAhead = 3;
-      u32x4_t af[kAhead];
+      // all sixteen K operand reads are written out up front; the scheduling directives below make
+      // the compiler keep kAhead of them in flight in front of the dependent MFMA chain instead of
+      // waiting for each read right before its MFMA
+      constexpr int kAhead = 4;
+      u32x4_t af[16];
 #pragma unroll
-      for (int s = 0; s < kAhead; s++)
-        af[s] = *reinterpret_cast<const u32x4_t*>(st + ((k_off ^ ((s & 7) << 5)) + (s >> 3) * 256));
+      for (int s2 = 0; s2 < 16; s2++)
+        af[s2] = *reinterpret_cast<const u32x4_t*>(st + ((k_off ^ ((s2 & 7) << 5)) + (s2 >> 3) * 256));
 #pragma unroll
-      for (int s = 0; s < 16; s++) {
-        u32x4_t cur = af[s % kAhead];
-        if (s + kAhead < 16) {
-          const int s2 = s + kAhead;
-          af[s % kAhead] = *reinterpret_cast<const u32x4_t*>(st + ((k_off ^ ((s2 & 7) << 5)) + (s2 >> 3) * 256));
-        }
-        sacc = mfma32<KDT>(cur, qf[s], sacc);
+      for (int s2 = 0; s2 < 16; s2++) sacc = mfma32<KDT>(af[s2], qf[s2], sacc);
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);  // DS reads
+#pragma unroll
+      for (int s2 = 0; s2 < 16 - kAhead; s2++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
     }
-
+  };
+  // stage 2 of a tile: online softmax on the vector units, then O^T += V^T . P^T on the matrix cores
+  auto softmax_pv_tile = [&](const unsigned char* st, int key0, f32x16_t& sacc) {
     // online softmax (log2 domain); register i is key key0 + 8 (i/4) + 4 g + i%4
+    // The maximum is tracked on the raw scores and the softmax scale (> 0) goes into the exponent's
+    // fused multiply-add, so a score costs one max, one fma and one exp2.
     float tmax = -__builtin_inff();
     if (key0 + kTile - 1 <= past + q0) {  // wave-uniform: no query of the wave masks any key of the tile
 #pragma unroll
-      for (int i = 0; i < 16; i++) {
-        sacc[i] *= a.scale_log2;
-        tmax = fmaxf(tmax, sacc[i]);
-      }
+      for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, sacc[i]);
     } else {
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         const bool valid = key0 + 8 * (i / 4) + 4 * g + (i % 4) <= qpos;
-        sacc[i] = valid ? sacc[i] * a.scale_log2 : -__builtin_inff();
+        sacc[i] = valid ? sacc[i] : -__builtin_inff();
         tmax = fmaxf(tmax, sacc[i]);
       }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, MSPR_WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, MSPR_WAVE)) * a.scale_log2;
     constexpr float kGrow = KDT == MSPR_BF16 ? 64.0f : 8.0f;
     const bool grow = tmax > m_run + kGrow;
     if (__any(grow)) {
@@ -270,11 +275,11 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
 #pragma unroll
       for (int mt = 0; mt < 8; mt++) oacc[mt] = oacc[mt] * alpha;
     }
-    const float m_safe = m_run == -__builtin_inff() ? 0.0f : m_run;
+    const float neg_m = m_run == -__builtin_inff() ? 0.0f : -m_run;
     float psum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
-      sacc[i] = __builtin_amdgcn_exp2f(sacc[i] - m_safe);
+      sacc[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[i], a.scale_log2, neg_m));
       psum += sacc[i];
     }
     l_run += psum;
@@ -284,19 +289,39 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
       pf[ks] = u32x4_t{pack2<KDT>(sacc[8 * ks], sacc[8 * ks + 1]), pack2<KDT>(sacc[8 * ks + 2], sacc[8 * ks + 3]),
                        pack2<KDT>(sacc[8 * ks + 4], sacc[8 * ks + 5]), pack2<KDT>(sacc[8 * ks + 6], sacc[8 * ks + 7])};
 
-    // O^T += V^T . P^T
+    // O^T += V^T . P^T; the transpose reads run kAheadV MFMAs in front of their use
+    {
+      constexpr int kAheadV = 4;
+      u32x4_t vf[16];
 #pragma unroll
-    for (int mt = 0; mt < 8; mt++) {
+      for (int mt = 0; mt < 8; mt++) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        const unsigned char* lo_p = st + ((v_off[0] ^ ((mt & 3) << 6)) + (mt >> 2) * 256 + ks * 16 * kRowBytes);
-        const unsigned char* hi_p = st + ((v_off[1] ^ ((mt & 3) << 6)) + (mt >> 2) * 256 + ks * 16 * kRowBytes);
-        s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, lo_p));
-        s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, hi_p));
-        u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
-        oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
+        for (int ks = 0; ks < 2; ks++) {
+          const unsigned char* lo_p = st + ((v_off[0] ^ ((mt & 3) << 6)) + (mt >> 2) * 256 + ks * 16 * kRowBytes);
+          const unsigned char* hi_p = st + ((v_off[1] ^ ((mt & 3) << 6)) + (mt >> 2) * 256 + ks * 16 * kRowBytes);
+          s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, lo_p));
+          s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, hi_p));
+          u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
+          vf[2 * mt + ks] = u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y};
+        }
       }
+#pragma unroll
+      for (int mt = 0; mt < 8; mt++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) oacc[mt] = mfma32<KDT>(vf[2 * mt + ks], pf[ks], oacc[mt]);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAheadV, 0);
+#pragma unroll
+      for (int i = 0; i < 16 - kAheadV; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAheadV, 0);
     }
+  };
+  auto compute_tile = [&](const unsigned char* st, int key0) {
+    f32x16_t sacc;
+    qk_tile(st, sacc);
+    softmax_pv_tile(st, key0, sacc);
   };
 
   if constexpr (Q8) {
@@ -360,17 +385,35 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   }
 
   // ---- dense tiles through the asynchronous ring: every wave issues its share of every tile
-  //      (clamped past the end), so the waits are static counts
+  //      (clamped past the end), so the waits are static counts.
+  // The two waves that share a SIMD run half a tile apart: waves 0-3 do both stages of tile t in
+  // iteration t, waves 4-7 do stage 2 of tile t-1 and then stage 1 of tile t, so that after the
+  // barrier the two are in different stages instead of queueing for the same unit. The late group
+  // still reads tile t-1 in iteration t, hence four ring slots.
   issue_tile(t1, 0);
   issue_tile(t1 + 1 < n_tiles ? t1 + 1 : n_tiles - 1, 1);
-  for (int t = t1; t < n_tiles; t++) {
-    // tile t has landed once this wave's copies of it are done (4 newer ones may be in flight) and
-    // every wave got here; the ring slot of tile t-1 is free after the barrier
-    wait_vm_and_barrier<4>();
-    issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - t1 + 2) % kBufs);  // past the end: a harmless re-read
-    const int key0 = t * kTile;
-    if (key0 > my_last_key) continue;  // wave-uniform: this wave's queries see none of the tile
-    compute_tile(lds + ((t - t1) % kBufs) * kStageBytes, key0);
+  if (Q8 || wave < 4) {  // (the quantised-prefix form keeps one schedule: its code is large enough already)
+    for (int t = t1; t < n_tiles; t++) {
+      // tile t has landed once this wave's copies of it are done (4 newer ones may be in flight) and
+      // every wave got here; the ring slot of tile t-2 is free after the barrier
+      wait_vm_and_barrier<4>();
+      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - t1 + 2) % kBufs);  // past the end: a harmless re-read
+      const int key0 = t * kTile;
+      if (key0 > my_last_key) continue;  // wave-uniform: this wave's queries see none of the tile
+      compute_tile(lds + ((t - t1) % kBufs) * kStageBytes, key0);
+    }
+  } else {
+    f32x16_t sacc;
+    bool pending = false;  // stage 2 of the previous tile still to do (wave-uniform)
+    for (int t = t1; t < n_tiles; t++) {
+      wait_vm_and_barrier<4>();
+      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - t1 + 2) % kBufs);
+      if (pending) softmax_pv_tile(lds + ((t - 1 - t1) % kBufs) * kStageBytes, (t - 1) * kTile, sacc);
+      const int key0 = t * kTile;
+      pending = key0 <= my_last_key;
+      if (pending) qk_tile(lds + ((t - t1) % kBufs) * kStageBytes, sacc);
+    }
+    if (pending) softmax_pv_tile(lds + ((n_tiles - 1 - t1) % kBufs) * kStageBytes, (n_tiles - 1) * kTile, sacc);
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped trailing copies must not outlive the workgroup's LDS
 

@@ -7,7 +7,7 @@
 // bf16 x bf16 product is exact in the float32 accumulator, so the only rounding is the
 // accumulation itself. Keys stream from HBM straight into the B-operand registers: a lane owns
 // 64 contiguous bytes of its key row, a wave 4 KB of contiguous memory per 32-key tile, and the
-// next tile is in flight while the current one is multiplied.
+// next two tiles are in flight while the current one is multiplied.
 #include "common.h"
 #include "profile.h"
 
@@ -40,6 +40,28 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
   const float* wb = weights + (int64_t)b * n_heads;
   float* sb = scores + (int64_t)b * n_rows;
 
+  const int64_t n_tiles = (n_rows + 31) / 32;
+  const int64_t stride = (int64_t)blocks_per_batch * 4;
+  int64_t tile = (int64_t)blk * 4 + wave;
+  if (tile >= n_tiles) return;
+
+  // a tile image: the lane's 64 key bytes and the key's scale (loaded with the tile so that the wait
+  // for it in the epilogue does not have to drain the tiles fetched behind it)
+  auto load_tile = [&](int64_t t, u32x4_t (&raw)[4], float& ks) {
+    int64_t row = t * 32 + m;
+    if (row >= n_rows) row = n_rows - 1;
+    ks = ksb[row];
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(kb + row * 128 + 64 * g);
+#pragma unroll
+    for (int j = 0; j < 4; j++) raw[j] = p[j];
+  };
+
+  // the first two tiles go out before anything else: their HBM latency overlaps the query loads
+  u32x4_t ra[4], rb[4], rc[4];
+  float sa, sb_, sc;
+  const int64_t last = n_tiles - 1;
+  load_tile(tile, ra, sa);
+  load_tile(tile + stride < n_tiles ? tile + stride : last, rb, sb_);
   // A operand: lane (m -> head, g) holds q[head][64g + 8s .. +7] for k-step s; heads past the end are zero
   u32x4_t qa[2][8];
 #pragma unroll
@@ -47,8 +69,11 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
     const int head = 32 * mt + m;
     const bool live = head < n_heads;
     const u32x4_t* p = reinterpret_cast<const u32x4_t*>(qb + (int64_t)(live ? head : 0) * 128 + 64 * g);
+    u32x4_t raw[8];
 #pragma unroll
-    for (int s = 0; s < 8; s++) qa[mt][s] = live ? p[s] : u32x4_t{0u, 0u, 0u, 0u};
+    for (int s = 0; s < 8; s++) raw[s] = p[s];  // unconditional (clamped) loads, selected afterwards
+#pragma unroll
+    for (int s = 0; s < 8; s++) qa[mt][s] = live ? raw[s] : u32x4_t{0u, 0u, 0u, 0u};
   }
   // weights of this lane's accumulator rows: head = 32mt + 8(i/4) + 4g + i%4
   float wl[2][16];
@@ -57,30 +82,12 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       const int head = 32 * mt + 8 * (i / 4) + 4 * g + (i % 4);
-      wl[mt][i] = head < n_heads ? wb[head] : 0.0f;
+      const float wv = wb[head < n_heads ? head : 0];
+      wl[mt][i] = head < n_heads ? wv : 0.0f;
     }
 
-  const int64_t n_tiles = (n_rows + 31) / 32;
-  const int64_t stride = (int64_t)blocks_per_batch * 4;
-  int64_t tile = (int64_t)blk * 4 + wave;
-  if (tile >= n_tiles) return;
-
-  auto load_tile = [&](int64_t t, u32x4_t (&raw)[4]) {
-    int64_t row = t * 32 + m;
-    if (row >= n_rows) row = n_rows - 1;
-    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(kb + row * 128 + 64 * g);
-#pragma unroll
-    for (int j = 0; j < 4; j++) raw[j] = p[j];
-  };
-
-  u32x4_t cur[4], nxt[4];
-  load_tile(tile, cur);
-  for (; tile < n_tiles; tile += stride) {
-    const bool more = tile + stride < n_tiles;
-    if (more) load_tile(tile + stride, nxt);
-    const int64_t row = tile * 32 + m;
-    const float ks = ksb[row < n_rows ? row : n_rows - 1];
-
+  auto compute_tile = [&](int64_t t, const u32x4_t (&cur)[4], float ks) {
+    const int64_t row = t * 32 + m;
     f32x16_t acc0 = {0}, acc1 = {0};
 #pragma unroll
     for (int s = 0; s < 8; s++) {
@@ -99,10 +106,23 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
     for (int i = 0; i < 16; i++) sum = fmaf(fmaxf(acc1[i], 0.0f), wl[1][i], sum);
     sum += __shfl_xor(sum, 32, MSPR_WAVE);
     if (g == 0 && row < n_rows) sb[row] = sum * ks;
-    if (more) {
-#pragma unroll
-      for (int j = 0; j < 4; j++) cur[j] = nxt[j];
-    }
+  };
+
+  // Three tile images rotate through registers: while one is multiplied the next two are in flight
+  // (8 KB per wave). Loads past the wave's last tile are clamped re-reads and are never consumed.
+  while (true) {
+    load_tile(tile + 2 * stride < n_tiles ? tile + 2 * stride : last, rc, sc);
+    compute_tile(tile, ra, sa);
+    tile += stride;
+    if (tile >= n_tiles) break;
+    load_tile(tile + 2 * stride < n_tiles ? tile + 2 * stride : last, ra, sa);
+    compute_tile(tile, rb, sb_);
+    tile += stride;
+    if (tile >= n_tiles) break;
+    load_tile(tile + 2 * stride < n_tiles ? tile + 2 * stride : last, rb, sb_);
+    compute_tile(tile, rc, sc);
+    tile += stride;
+    if (tile >= n_tiles) break;
   }
 }
 

@@ -644,17 +644,11 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   const int64_t part0 = (int64_t)(seq * a.n_hblk + hb) * a.n_splits;
   const float* ml0 = a.ws_ml + (part0 * 64 + hg * 32 + n) * 2;
   const float* wo0 = a.ws_o + (part0 * 4 + wave) * (int64_t)(8 * 16 * 64) + ((mt * 4 + c) * 64 + lane) * 4;
-  constexpr int kChunk = 8;
-  float m_all = sink;
-  for (int s0 = 0; s0 < a.n_splits; s0 += kChunk) {
-    float mv[kChunk];
-#pragma unroll
-    for (int j = 0; j < kChunk; j++) mv[j] = s0 + j < a.n_splits ? ml0[(int64_t)(s0 + j) * 128] : -__builtin_inff();
-#pragma unroll
-    for (int j = 0; j < kChunk; j++) m_all = fmaxf(m_all, mv[j]);
-  }
-  const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
-  float l = exp2f(sink - m_safe);
+  // One online pass in chunks of 16 ranges: the statistics and the partial rows of a chunk are all
+  // requested at once, so a sequence split into up to 16 ranges costs one memory round trip.
+  constexpr int kChunk = 16;
+  float m_run = sink;  // the sink joins the maximum and the denominator once
+  float l = sink == -__builtin_inff() ? 0.0f : 1.0f;
   f32x4_t o = {0.f, 0.f, 0.f, 0.f};
   for (int s0 = 0; s0 < a.n_splits; s0 += kChunk) {
     float mv[kChunk], lv[kChunk];
@@ -663,16 +657,25 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
     for (int j = 0; j < kChunk; j++) {
       const bool live = s0 + j < a.n_splits;
       const int64_t sj = live ? s0 + j : 0;
-      mv[j] = live ? ml0[sj * 128] : -__builtin_inff();
+      mv[j] = ml0[sj * 128];
       lv[j] = ml0[sj * 128 + 1];
       ov[j] = *reinterpret_cast<const f32x4_t*>(wo0 + sj * (int64_t)(4 * 8 * 16 * 64));
+      if (!live) mv[j] = -__builtin_inff();
     }
+    float m_new = m_run;
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) m_new = fmaxf(m_new, mv[j]);
+    const float m_safe = m_new == -__builtin_inff() ? 0.0f : m_new;
+    const float alpha = fast_exp2(m_run - m_safe);  // 0 while nothing has been accumulated
+    l *= alpha;
+    o = o * alpha;
 #pragma unroll
     for (int j = 0; j < kChunk; j++) {
-      float w = exp2f(mv[j] - m_safe);
+      const float w = fast_exp2(mv[j] - m_safe);
       l += lv[j] * w;
       o += ov[j] * w;
     }
+    m_run = m_new;
   }
   const float inv = l == 0.0f ? 0.0f : 1.0f / l;
   float r[4] = {o.x * inv, o.y * inv, o.z * inv, o.w * inv};
