@@ -222,10 +222,10 @@ struct Geometry {
   static constexpr int kSxBytes = 4 * 16 * 64 * 4; // 4 waves x 16 floats x 64 lanes
   static constexpr int kMaxIds = 1024;             // gathered slots per workgroup
   static constexpr int kOffSx = kBufs * kTileBytes;
-  static constexpr int kOffRowPtr = kOffSx + 2 * kSxBytes;
-  static constexpr int kOffVmask = kOffRowPtr + kBufs * kTile * 8;
-  static constexpr int kOffIds = kOffVmask + 16;
-  static constexpr int kOffRope = kOffIds + kMaxIds * 4;
+  static constexpr int kMaxTiles = kMaxIds / kTile; // tiles per workgroup (slots_per_split <= kMaxIds)
+  static constexpr int kOffRowPtr = kOffSx + 2 * kSxBytes;       // row pointer of every slot of the workgroup
+  static constexpr int kOffVmask = kOffRowPtr + kMaxIds * 8;     // one validity word per tile
+  static constexpr int kOffRope = kOffVmask + kMaxTiles * 4;
   static constexpr int kOffStop = kOffRope + 64 * 4;
   static constexpr int kLdsBytes = kOffStop + 16;
   static_assert(kInstr % 4 == 1, "wave 0 issues exactly one load more than the other waves");
@@ -237,9 +237,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   unsigned char* kbuf = lds;                                                   // [kBufs][kTileBytes]
   float* sx = reinterpret_cast<float*>(lds + G::kOffSx);                       // [2][4][16*64]
-  uint64_t* rowptr = reinterpret_cast<uint64_t*>(lds + G::kOffRowPtr);         // [kBufs][kTile]
-  uint32_t* vmask = reinterpret_cast<uint32_t*>(lds + G::kOffVmask);           // [4]
-  int32_t* ids = reinterpret_cast<int32_t*>(lds + G::kOffIds);                 // [kMaxIds]
+  uint64_t* rowptr = reinterpret_cast<uint64_t*>(lds + G::kOffRowPtr);         // [kMaxIds]
+  uint32_t* vmask = reinterpret_cast<uint32_t*>(lds + G::kOffVmask);           // [kMaxTiles]
   float* rope_c = reinterpret_cast<float*>(lds + G::kOffRope);
   float* rope_s = rope_c + 32;
   int* stop_shared = reinterpret_cast<int*>(lds + G::kOffStop);
@@ -292,13 +291,22 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   const int32_t* idx_b = a.idx + (int64_t)seq * a.idx_batch_stride;
 
   MSPR_STAMP(0);
-  // ---- query operand loads go out first: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7]
+  // ---- query operand: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7]; its loads go out
+  //      right behind the id loads below and are back by the time the row pointer table is built
   const int head = hb * 64 + hg * 32 + n;
   const bool q_live = head < a.n_heads;
   const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)t * a.q_token_stride +
                        (int64_t)(q_live ? head : 0) * a.q_head_stride + dh * G::kHalf + 8 * g;
   u32x4_t qf[G::kSteps];
   f32x4_t qraw32[QDT == MSPR_F32 ? G::kSteps : 1][2];
+  // The gathered ids of this thread's slots are requested before anything else: ids -> row pointers ->
+  // rows is the longest dependency chain of the prologue. Slot ls = tid + 256 j of the range.
+  int my_id[G::kMaxIds / kThreads];
+#pragma unroll
+  for (int j = 0; j < G::kMaxIds / kThreads; j++) {
+    const int gi = slot0 + tid + kThreads * j - seq_n_win;
+    my_id[j] = (gi >= 0 && gi < a.n_idx && j * kThreads < n_tiles * kTile) ? idx_b[gi] : -1;
+  }
   if constexpr (QDT == MSPR_F32) {
     const float* qp = reinterpret_cast<const float*>(a.q) + qoff;
 #pragma unroll
@@ -311,6 +319,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 #pragma unroll
     for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = *reinterpret_cast<const u32x4_t*>(qp + 16 * ks);
   }
+
 
   // ---- stop position of the gathered walk, rope table, gathered ids of this slot range
   if (ROPE && tid < 32) {
@@ -332,10 +341,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     stop_pos = *stop_shared;
   }
   const int subst_slot = a.subst_from_params ? a.params[1] : a.subst_slot;
-  const int id_base = slot0 > seq_n_win ? slot0 - seq_n_win : 0;           // first gathered index of the range
-  const int id_count = slot1 > seq_n_win ? slot1 - seq_n_win - id_base : 0;  // <= kMaxIds by construction
-  for (int i = tid; i < id_count; i += kThreads) ids[i] = id_base + i < stop_pos ? idx_b[id_base + i] : -1;
-
   // ---- static part of this thread's tile loads: LDS slot P = tid + 256 j holds (row P / kSlots, chunk P % kSlots)
   uint32_t pk[G::kPerThread];
 #pragma unroll
@@ -346,9 +351,15 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   }
   const uint64_t zero_row = reinterpret_cast<uint64_t>(&g_zero_row[0]);
 
-  // row pointers and validity of one tile (32 lanes of one half-wave)
-  auto fill_rows = [&](int tile, int l32, uint64_t ballot_shift) {
-    const int slot = slot0 + tile * kTile + l32;
+  // ---- row pointer and validity of every slot of this workgroup's range, by all threads at once:
+  //      window slots map to ring rows (or the substituted row), gathered slots read their id from
+  //      global memory; skipped slots point at a zero row so that every tile load stays fully active
+#pragma unroll
+  for (int tj = 0; tj < G::kMaxIds / kThreads; tj++) {
+    const int s0 = tj * kThreads;
+    if (s0 >= n_tiles * kTile) break;
+    const int ls = s0 + tid;  // slot inside the range (the loop bound is a multiple of 32, whole waves or half waves run)
+    const int slot = slot0 + ls;
     uint64_t ptr = zero_row;
     bool valid = false;
     if (slot < slot1) {
@@ -361,7 +372,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
           ptr = reinterpret_cast<uint64_t>(win_b + (int64_t)r * DK);
         }
       } else {
-        const int id = ids[slot - seq_n_win - id_base];
+        const int gi = slot - seq_n_win;  // index into the gathered id list
+        const int id = gi < stop_pos ? my_id[tj] : -1;
         if (id >= 0) {
           const int64_t r = (int64_t)id * a.row_mul + a.row_add;
           if (r >= 0 && r < a.n_pool) {
@@ -371,18 +383,16 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         }
       }
     }
-    rowptr[(tile % G::kBufs) * kTile + l32] = ptr;
     const uint64_t bal = __ballot(valid);
-    if (l32 == 0) vmask[tile & 3] = (uint32_t)(bal >> ballot_shift);
-  };
-  // asynchronous loads of one tile straight into its LDS ring buffer
-  auto issue_tile = [&](int tile) {
-    const int buf = tile % G::kBufs;
-    const uint64_t* rp = rowptr + buf * kTile;
-    const uint32_t dst_lds = __builtin_amdgcn_readfirstlane(
-        (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, kbuf + buf * G::kTileBytes + wave * 1024));
-    // all row pointers first (the asm statements below are compiler barriers for memory operations)
-    uint64_t src[G::kPerThread];
+    if (ls < n_tiles * kTile) {
+      rowptr[ls] = ptr;
+      if ((lane & 31) == 0) vmask[ls >> 5] = (uint32_t)(bal >> (lane & 32));
+    }
+  }
+  // asynchronous loads of one tile straight into its LDS ring buffer: source addresses first (LDS
+  // reads of the row pointers), then one 1 KB copy per call of issue_one
+  auto tile_sources = [&](int tile, uint64_t (&src)[G::kPerThread]) {
+    const uint64_t* rp = rowptr + tile * kTile;
 #pragma unroll
     for (int j = 0; j < G::kPerThread; j++) {
       const uint32_t p = pk[j];
@@ -390,18 +400,26 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       // lanes of the padding slot fetch a harmless duplicate so that every load is fully active
       src[j] = rp[act ? (p >> 16) : 0] + (act ? (p & 0xFFFFu) : 0u);
     }
+  };
+  auto tile_lds_base = [&](int tile) -> uint32_t {
+    return __builtin_amdgcn_readfirstlane(
+        (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, kbuf + (tile % G::kBufs) * G::kTileBytes + wave * 1024));
+  };
+  auto issue_one = [&](const uint64_t (&src)[G::kPerThread], uint32_t dst_lds, int j) {
+    if (j < G::kPerThread - 1 || wave == 0) async_load_16(src[j], dst_lds + j * 4096);
+  };
+  auto issue_tile = [&](int tile) {
+    uint64_t src[G::kPerThread];
+    tile_sources(tile, src);
+    const uint32_t dst_lds = tile_lds_base(tile);
 #pragma unroll
-    for (int j = 0; j < G::kPerThread; j++) {
-      if (j < G::kPerThread - 1 || wave == 0) async_load_16(src[j], dst_lds + j * 4096);
-    }
+    for (int j = 0; j < G::kPerThread; j++) issue_one(src, dst_lds, j);
   };
 
-  __syncthreads();  // ids visible
   MSPR_STAMP(1);
-  if (tid < 96 && tid / 32 < n_tiles) fill_rows(tid / 32, tid & 31, (tid & 32) ? 32 : 0);
-  lds_barrier();
-  // The query loads must be complete before the first asynchronous tile load goes out: a wait left
-  // for their first use would otherwise also wait for (drain) the tile loads behind them.
+  __syncthreads();  // row pointer table visible
+  // The query loads (issued long ago) must be complete before the first asynchronous tile load goes
+  // out: a wait left for their first use would otherwise also wait for (drain) the tile loads behind them.
   if constexpr (QDT == MSPR_F32) {
 #pragma unroll
     for (int ks = 0; ks < G::kSteps; ks++) asm volatile("" : "+v"(qraw32[ks][0]), "+v"(qraw32[ks][1]));
@@ -477,11 +495,19 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       wait_vm_and_barrier<0>();
     }
     MSPR_STAMP(4 + 6 * t);
-    if (t + 2 < n_tiles) issue_tile(t + 2);  // its ring buffer held tile t-1, which every wave has left
-    if (t + 3 < n_tiles && tid < 32) fill_rows(t + 3, tid, 0);
+    // tile t+2 goes into the ring buffer of tile t-1, which every wave has left; its copies are issued
+    // between the matrix-core instructions below, so that the time a copy waits for the address unit
+    // is covered by MFMAs already in flight
+    const bool more = t + 2 < n_tiles;  // workgroup-uniform
+    uint64_t nsrc[G::kPerThread];
+    uint32_t ndst = 0;
+    if (more) {
+      tile_sources(t + 2, nsrc);
+      ndst = tile_lds_base(t + 2);
+    }
     const int buf = t % G::kBufs;
     const unsigned char* kt = kbuf + buf * G::kTileBytes;
-    const uint32_t mask_all = vmask[t & 3];
+    const uint32_t mask_all = vmask[t];
 
     MSPR_STAMP(5 + 6 * t);
     // S^T partial over this wave's half of the row width
@@ -497,7 +523,15 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         if (ks + kAhead < G::kSteps)
           af[ks % kAhead] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + (ks + kAhead) * 32);
         sacc = mfma32<KDT>(cur, qf[ks], sacc);
+        if (more && (ks & 1) == 0 && ks / 2 < G::kPerThread) {
+          issue_one(nsrc, ndst, ks / 2);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+    }
+    if (more) {
+#pragma unroll
+      for (int j = (G::kSteps + 1) / 2; j < G::kPerThread; j++) issue_one(nsrc, ndst, j);
     }
     float* sxw = sx + ((t & 1) * 4 + wave) * (16 * 64);
 #pragma unroll
