@@ -224,10 +224,16 @@ int mspr_sdpa_decode_q8_0(const void* queries, int q_dtype, const void* k_codes,
  * same dtype, rows [0, past_len+q_len) valid; n_q_heads/n_kv_heads in {1,2,4,8}. */
 int mspr_flash_prefill(const void* q, const void* k, const void* v, int dtype, int batch, int n_q_heads,
                        int n_kv_heads, int head_dim, int q_len, int64_t past_len, int64_t kv_rows,
-                       float scale, void* out, void* stream);
+                       float scale, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Workspace bytes of mspr_sdpa_fa_prefill_q8 (float16 copies of the chunk's own K/V rows). */
-size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_kv_heads, int q_len, int64_t past_len);
+/* Workspace bytes of mspr_flash_prefill (key-range partials of short chunks; 256 when none are needed). */
+size_t mspr_flash_prefill_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len,
+                                          int64_t past_len);
+
+/* Workspace bytes of mspr_sdpa_fa_prefill_q8 (float16 copies of the chunk's own K/V rows, plus the
+ * key-range partials when a short chunk over a deep prefix is split to fill the device). */
+size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len,
+                                               int64_t past_len);
 
 /* Causal flash prefill over an affine 8-bit prefix plus the dense chunk itself: query row i attends
  * every prefix key and chunk keys [0, i].

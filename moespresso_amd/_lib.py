@@ -66,8 +66,9 @@ SIGNATURES = {
                 c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_flash_prefill": (
         c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_float,
-                c_void_p, c_void_p]),
-    "mspr_sdpa_fa_prefill_q8_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int64]),
+                c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mspr_flash_prefill_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int64]),
+    "mspr_sdpa_fa_prefill_q8_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int64]),
     "mspr_sdpa_fa_prefill_q8": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                 c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p, c_void_p,

@@ -37,6 +37,11 @@ struct PrefillArgs {
   float scale_log2;
   int rep_shift;    // log2(query heads per KV head), 0..3
   int q_blocks;     // workgroups along the query axis
+  // key-range splits (short chunks over deep prefixes do not fill the device otherwise): split sp of a
+  // query block takes every n_splits-th share of that block's tiles; partials are merged afterwards
+  int n_splits;
+  float* ws_o;      // [n_splits][B][Hq][L][256] unnormalised O relative to ws_ml's maximum
+  float* ws_ml;     // [n_splits][B][Hq][L][2]   (reference maximum in log2 units, denominator)
   // quantised-prefix form only: tiles [0, q8_tiles) come from the affine 8-bit prefix below, the rest
   // from k / v, which then hold float16 rows for keys [32 q8_tiles, past_len + q_len)
   int q8_tiles;
@@ -130,6 +135,8 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   const int sub_blocks = 8 >> a.rep_shift;  // 32-row query sub-blocks per workgroup
   const int rows_per_wg = 32 * sub_blocks;
   int work = blockIdx.x;
+  const int sp = work % a.n_splits;
+  work /= a.n_splits;
   const int qb = a.q_blocks - 1 - work % a.q_blocks;
   work /= a.q_blocks;
   const int kvh = work % a.n_kv_heads;
@@ -146,7 +153,11 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   // keys needed by the workgroup: [0, past + last query row]
   int q_last = qb * rows_per_wg + rows_per_wg - 1;
   if (q_last > a.q_len - 1) q_last = a.q_len - 1;
-  const int n_tiles = (int)((past + q_last) / kTile) + 1;
+  const int all_tiles = (int)((past + q_last) / kTile) + 1;
+  // this workgroup's share of the block's tiles: [t_begin, n_tiles)
+  const int tiles_per_split = (all_tiles + a.n_splits - 1) / a.n_splits;
+  const int t_begin = sp * tiles_per_split < all_tiles ? sp * tiles_per_split : all_tiles;
+  const int n_tiles = t_begin + tiles_per_split < all_tiles ? t_begin + tiles_per_split : all_tiles;
 
   // ---- asynchronous tile copies: thread handles LDS slots tid and tid + 512 of the K and of the V tile;
   //      addresses are a scalar tile base plus a per-thread 32-bit offset
@@ -327,7 +338,8 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   if constexpr (Q8) {
     // ---- quantised prefix: tile t+1 is unpacked from registers into the other LDS slot at the top of
     //      step t while the raw bytes of tile t+2 are already on their way
-    if (t1 > 0) {
+    const int p_end = n_tiles < t1 ? n_tiles : t1;  // prefix tiles of this workgroup: [t_begin, p_end)
+    if (t_begin < p_end) {
       const int s_row = tid >> 4;   // tile row staged by this thread
       const int s_pp = tid & 15;    // its 16 elements: [16 s_pp, +16), scale group s_pp / 4
       const int64_t row0 = ((int64_t)b * a.n_kv_heads + kvh) * past;
@@ -369,16 +381,16 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
         *reinterpret_cast<u32x4_t*>(st + kTileBytes + w_off0) = p0;
         *reinterpret_cast<u32x4_t*>(st + kTileBytes + w_off1) = p1;
       };
-      load_raw(0);
+      load_raw(t_begin);
       unpack_to(0);
-      if (t1 > 1) load_raw(1);
-      for (int t = 0; t < t1; t++) {
+      if (t_begin + 1 < p_end) load_raw(t_begin + 1);
+      for (int t = t_begin; t < p_end; t++) {
         __syncthreads();  // tile t is complete in LDS; every wave has left tile t-1
-        if (t + 1 < t1) {
-          unpack_to((t + 1) & 1);
-          if (t + 2 < t1) load_raw(t + 2);
+        if (t + 1 < p_end) {
+          unpack_to((t + 1 - t_begin) & 1);
+          if (t + 2 < p_end) load_raw(t + 2);
         }
-        compute_tile(lds + (t & 1) * kStageBytes, t * kTile);
+        compute_tile(lds + ((t - t_begin) & 1) * kStageBytes, t * kTile);
       }
       __syncthreads();  // every wave has left the last prefix tile before the ring below reuses the slots
     }
@@ -390,35 +402,55 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   // iteration t, waves 4-7 do stage 2 of tile t-1 and then stage 1 of tile t, so that after the
   // barrier the two are in different stages instead of queueing for the same unit. The late group
   // still reads tile t-1 in iteration t, hence four ring slots.
-  issue_tile(t1, 0);
-  issue_tile(t1 + 1 < n_tiles ? t1 + 1 : n_tiles - 1, 1);
+  const int r0 = t_begin > t1 ? t_begin : t1;  // first tile of this workgroup that is served from k / v
+  if (r0 < n_tiles) {
+  issue_tile(r0, 0);
+  issue_tile(r0 + 1 < n_tiles ? r0 + 1 : n_tiles - 1, 1);
   if (Q8 || wave < 4) {  // (the quantised-prefix form keeps one schedule: its code is large enough already)
-    for (int t = t1; t < n_tiles; t++) {
+    for (int t = r0; t < n_tiles; t++) {
       // tile t has landed once this wave's copies of it are done (4 newer ones may be in flight) and
       // every wave got here; the ring slot of tile t-2 is free after the barrier
       wait_vm_and_barrier<4>();
-      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - t1 + 2) % kBufs);  // past the end: a harmless re-read
+      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - r0 + 2) % kBufs);  // past the end: a harmless re-read
       const int key0 = t * kTile;
       if (key0 > my_last_key) continue;  // wave-uniform: this wave's queries see none of the tile
-      compute_tile(lds + ((t - t1) % kBufs) * kStageBytes, key0);
+      compute_tile(lds + ((t - r0) % kBufs) * kStageBytes, key0);
     }
   } else {
     f32x16_t sacc;
     bool pending = false;  // stage 2 of the previous tile still to do (wave-uniform)
-    for (int t = t1; t < n_tiles; t++) {
+    for (int t = r0; t < n_tiles; t++) {
       wait_vm_and_barrier<4>();
-      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - t1 + 2) % kBufs);
-      if (pending) softmax_pv_tile(lds + ((t - 1 - t1) % kBufs) * kStageBytes, (t - 1) * kTile, sacc);
+      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - r0 + 2) % kBufs);
+      if (pending) softmax_pv_tile(lds + ((t - 1 - r0) % kBufs) * kStageBytes, (t - 1) * kTile, sacc);
       const int key0 = t * kTile;
       pending = key0 <= my_last_key;
-      if (pending) qk_tile(lds + ((t - t1) % kBufs) * kStageBytes, sacc);
+      if (pending) qk_tile(lds + ((t - r0) % kBufs) * kStageBytes, sacc);
     }
-    if (pending) softmax_pv_tile(lds + ((n_tiles - 1 - t1) % kBufs) * kStageBytes, (n_tiles - 1) * kTile, sacc);
+    if (pending) softmax_pv_tile(lds + ((n_tiles - 1 - r0) % kBufs) * kStageBytes, (n_tiles - 1) * kTile, sacc);
+  }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped trailing copies must not outlive the workgroup's LDS
 
   // ---- normalise and store: lane (n, g) holds dims 32 mt + 8 (i/4) + 4 g + i%4 of query row q0 + n
   const float l_tot = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
+  if (a.n_splits > 1) {
+    if (q0 + n < a.q_len) {
+      const int64_t row = (((int64_t)sp * a.batch + b) * a.n_q_heads + head) * a.q_len + q0 + n;
+      float* po = a.ws_o + row * kD;
+#pragma unroll
+      for (int mt = 0; mt < 8; mt++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          *reinterpret_cast<f32x4_t*>(po + 32 * mt + 8 * c + 4 * g) =
+              f32x4_t{oacc[mt][4 * c], oacc[mt][4 * c + 1], oacc[mt][4 * c + 2], oacc[mt][4 * c + 3]};
+      if (g == 0) {
+        a.ws_ml[row * 2] = m_run;
+        a.ws_ml[row * 2 + 1] = l_tot;
+      }
+    }
+    return;
+  }
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
   if (q0 + n < a.q_len) {
     const int64_t ooff = (((int64_t)b * a.n_q_heads + head) * a.q_len + q0 + n) * kD;
@@ -475,6 +507,77 @@ __global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, con
   tail_v[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(vx);
 }
 
+// Merge of the key-range partials of one query row: 64 lanes x 4 columns, four rows per workgroup.
+template <int ODT>
+__global__ __launch_bounds__(256) void prefill_merge_kernel(PrefillArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t n_rows = (int64_t)a.batch * a.n_q_heads * a.q_len;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  float m_run = -__builtin_inff(), l = 0.0f;
+  f32x4_t o = {0.f, 0.f, 0.f, 0.f};
+  constexpr int kChunk = 8;
+  for (int s0 = 0; s0 < a.n_splits; s0 += kChunk) {
+    float mv[kChunk], lv[kChunk];
+    f32x4_t ov[kChunk];
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) {
+      const int sj = s0 + j < a.n_splits ? s0 + j : 0;
+      const int64_t r = (int64_t)sj * n_rows + row;
+      mv[j] = a.ws_ml[r * 2];
+      lv[j] = a.ws_ml[r * 2 + 1];
+      ov[j] = *reinterpret_cast<const f32x4_t*>(a.ws_o + r * kD + 4 * lane);
+      // a range that saw no key of this row contributes nothing (its O is whatever the registers held)
+      if (s0 + j >= a.n_splits || !(lv[j] > 0.0f)) {
+        mv[j] = -__builtin_inff();
+        lv[j] = 0.0f;
+        ov[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    float m_new = m_run;
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) m_new = fmaxf(m_new, mv[j]);
+    const float m_safe = m_new == -__builtin_inff() ? 0.0f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    l *= alpha;
+    o = o * alpha;
+#pragma unroll
+    for (int j = 0; j < kChunk; j++) {
+      const float w = __builtin_amdgcn_exp2f(mv[j] - m_safe);
+      l += lv[j] * w;
+      o += ov[j] * w;
+    }
+    m_run = m_new;
+  }
+  const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+  if constexpr (ODT == MSPR_F32) {
+    *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.out) + row * kD + 4 * lane) = o * inv;
+  } else {
+    u32x2_t w = {pack2<ODT>(o.x * inv, o.y * inv), pack2<ODT>(o.z * inv, o.w * inv)};
+    *reinterpret_cast<u32x2_t*>(reinterpret_cast<uint16_t*>(a.out) + row * kD + 4 * lane) = w;
+  }
+}
+
+// enough workgroups for the 256 CUs, at least 16 tiles (512 keys) per range
+int prefill_choose_splits(int batch, int n_kv_heads, int q_blocks, int64_t past_len, int q_len) {
+  const int64_t wgs = (int64_t)batch * n_kv_heads * q_blocks;
+  if (wgs >= 192) return 1;
+  int64_t want = (256 + wgs - 1) / wgs;
+  const int64_t tiles = (past_len + q_len + kTile - 1) / kTile;
+  if (want > tiles / 16) want = tiles / 16;
+  if (want > 32) want = 32;
+  return want < 1 ? 1 : (int)want;
+}
+
+size_t prefill_split_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len, int64_t past_len) {
+  const int rep = n_q_heads / n_kv_heads;
+  const int rows_per_wg = 32 * (8 / rep);
+  const int q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
+  const int splits = prefill_choose_splits(batch, n_kv_heads, q_blocks, past_len, q_len);
+  if (splits == 1) return 0;
+  return (size_t)splits * batch * n_q_heads * q_len * (kD + 2) * sizeof(float);
+}
+
 template <int KDT, bool Q8, int SDT>
 int prefill_launch(const PrefillArgs& a, hipStream_t st) {
   static bool attr_set = false;
@@ -487,20 +590,35 @@ int prefill_launch(const PrefillArgs& a, hipStream_t st) {
     }
     attr_set = true;
   }
-  dim3 grid((unsigned)(a.q_blocks * a.n_kv_heads * a.batch)), block(kThreads);
+  dim3 grid((unsigned)(a.q_blocks * a.n_kv_heads * a.batch * a.n_splits)), block(kThreads);
   {
     MsprProfScope prof(MSPR_K_FLASH_PREFILL, st);
     flash_prefill_kernel<KDT, Q8, SDT><<<grid, block, kLdsBytes, st>>>(a);
   }
   MSPR_CHECK_LAUNCH("flash_prefill");
+  if (a.n_splits > 1) {
+    const int64_t n_rows = (int64_t)a.batch * a.n_q_heads * a.q_len;
+    dim3 mgrid((unsigned)((n_rows + 3) / 4)), mblock(256);
+    if (Q8) prefill_merge_kernel<MSPR_F32><<<mgrid, mblock, 0, st>>>(a);
+    else prefill_merge_kernel<KDT><<<mgrid, mblock, 0, st>>>(a);
+    MSPR_CHECK_LAUNCH("flash_prefill (merge)");
+  }
   return MSPR_OK;
 }
 
 }  // namespace
 
+extern "C" size_t mspr_flash_prefill_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len,
+                                                     int64_t past_len) {
+  if (batch < 1 || n_kv_heads < 1 || n_q_heads < n_kv_heads || n_q_heads % n_kv_heads != 0 || q_len < 1 ||
+      past_len < 0 || n_q_heads / n_kv_heads > 8)
+    return 0;
+  return prefill_split_bytes(batch, n_q_heads, n_kv_heads, q_len, past_len) + 256;
+}
+
 extern "C" int mspr_flash_prefill(const void* q, const void* k, const void* v, int dtype, int batch, int n_q_heads,
                                   int n_kv_heads, int head_dim, int q_len, int64_t past_len, int64_t kv_rows,
-                                  float scale, void* out, void* stream) {
+                                  float scale, void* out, void* workspace, size_t workspace_bytes, void* stream) {
   MSPR_REQUIRE(q && k && v && out, "flash_prefill: null pointer");
   MSPR_REQUIRE(dtype == MSPR_BF16 || dtype == MSPR_F16, "flash_prefill: dtype must be float16 or bfloat16");
   MSPR_REQUIRE(head_dim == kD, "flash_prefill: head_dim must be 256");
@@ -528,16 +646,28 @@ extern "C" int mspr_flash_prefill(const void* q, const void* k, const void* v, i
   a.rep_shift = rep == 1 ? 0 : rep == 2 ? 1 : rep == 4 ? 2 : 3;
   const int rows_per_wg = 32 * (8 / rep);
   a.q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
-  MSPR_REQUIRE((int64_t)a.q_blocks * n_kv_heads * batch < ((int64_t)1 << 31), "flash_prefill: grid too large");
+  a.n_splits = prefill_choose_splits(batch, n_kv_heads, a.q_blocks, past_len, q_len);
+  MSPR_REQUIRE((int64_t)a.q_blocks * n_kv_heads * batch * a.n_splits < ((int64_t)1 << 31), "flash_prefill: grid too large");
+  if (a.n_splits > 1) {
+    const size_t need = prefill_split_bytes(batch, n_q_heads, n_kv_heads, q_len, past_len);
+    MSPR_REQUIRE(workspace && workspace_bytes >= need && mspr_aligned(workspace, 16),
+                 "flash_prefill: workspace of %zu bytes (16-byte aligned) needed, %zu given", need, workspace_bytes);
+    a.ws_o = reinterpret_cast<float*>(workspace);
+    a.ws_ml = a.ws_o + (size_t)a.n_splits * batch * n_q_heads * q_len * kD;
+  }
   hipStream_t st = (hipStream_t)stream;
   if (dtype == MSPR_BF16) return prefill_launch<MSPR_BF16, false, MSPR_F32>(a, st);
   return prefill_launch<MSPR_F16, false, MSPR_F32>(a, st);
 }
 
-extern "C" size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_kv_heads, int q_len, int64_t past_len) {
-  if (batch < 1 || n_kv_heads < 1 || q_len < 1 || past_len < 0) return 0;
+extern "C" size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len,
+                                                          int64_t past_len) {
+  if (batch < 1 || n_kv_heads < 1 || n_q_heads < n_kv_heads || n_q_heads % n_kv_heads != 0 || q_len < 1 ||
+      past_len < 0 || n_q_heads / n_kv_heads > 8)
+    return 0;
   const int64_t tail_rows = past_len % kTile + q_len;
-  return (size_t)batch * n_kv_heads * tail_rows * kRowBytes * 2 + 256;
+  const size_t tail = ((size_t)batch * n_kv_heads * tail_rows * kRowBytes * 2 + 255) / 256 * 256;
+  return tail + prefill_split_bytes(batch, n_q_heads, n_kv_heads, q_len, past_len) + 256;
 }
 
 extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, const void* pk_scales,
@@ -562,7 +692,7 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
                "sdpa_fa_prefill_q8: need q_len >= 1 and past_len >= 0");
   MSPR_REQUIRE(mspr_aligned(queries, 16) && mspr_aligned(out, 16) && mspr_aligned(pk_wq, 16) && mspr_aligned(pv_wq, 16),
                "sdpa_fa_prefill_q8: pointers must be 16-byte aligned");
-  const size_t need = mspr_sdpa_fa_prefill_q8_workspace_bytes(batch, n_kv_heads, q_len, past_len);
+  const size_t need = mspr_sdpa_fa_prefill_q8_workspace_bytes(batch, n_q_heads, n_kv_heads, q_len, past_len);
   MSPR_REQUIRE(workspace && workspace_bytes >= need && mspr_aligned(workspace, 16),
                "sdpa_fa_prefill_q8: workspace of %zu bytes (16-byte aligned) needed, %zu given", need, workspace_bytes);
   PrefillArgs a = {};
@@ -584,6 +714,12 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
   const int rows_per_wg = 32 * (8 / rep);
   a.q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
   a.q8_tiles = (int)(past_len / kTile);
+  a.n_splits = prefill_choose_splits(batch, n_kv_heads, a.q_blocks, past_len, q_len);
+  if (a.n_splits > 1) {
+    const size_t tail = ((size_t)batch * n_kv_heads * tail_rows * kRowBytes * 2 + 255) / 256 * 256;
+    a.ws_o = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + tail);
+    a.ws_ml = a.ws_o + (size_t)a.n_splits * batch * n_q_heads * q_len * kD;
+  }
   a.pk_wq = pk_wq;
   a.pk_s = pk_scales;
   a.pk_b = pk_biases;

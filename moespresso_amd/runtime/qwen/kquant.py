@@ -280,7 +280,7 @@ def sdpa_fa_prefill_q8(queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, p
         t.contiguous() for t in (queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, pv_biases, self_k, self_v)]
     out = torch.empty_like(q)
     if workspace is None:
-        nbytes = int(_lib.lib().mspr_sdpa_fa_prefill_q8_workspace_bytes(B, Hkv, L, P))
+        nbytes = int(_lib.lib().mspr_sdpa_fa_prefill_q8_workspace_bytes(B, Hq, Hkv, L, P))
         workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=q.device)
     _lib.check(_lib.lib().mspr_sdpa_fa_prefill_q8(
         _lib.ptr(q), _lib.ptr(kw), _lib.ptr(ks), _lib.ptr(kb), _lib.ptr(vw), _lib.ptr(vs), _lib.ptr(vb),
@@ -290,7 +290,7 @@ def sdpa_fa_prefill_q8(queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, p
     return out
 
 
-def flash_prefill(queries, keys, values, scale, *, past_len: int):
+def flash_prefill(queries, keys, values, scale, *, past_len: int, workspace=None):
     """Causal chunked-prefill GQA attention over a dense 16-bit cache that already holds the chunk.
 
     Query row ``i`` sits at position ``past_len + i`` and attends keys ``[0, past_len + i]``: the
@@ -324,7 +324,11 @@ def flash_prefill(queries, keys, values, scale, *, past_len: int):
     _lib.require_device(queries, keys, values)
     q, k, v = queries.contiguous(), keys.contiguous(), values.contiguous()
     out = torch.empty_like(q)
+    if workspace is None:
+        nbytes = int(_lib.lib().mspr_flash_prefill_workspace_bytes(B, Hq, Hkv, L, past_len))
+        workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=q.device)
     _lib.check(_lib.lib().mspr_flash_prefill(
         _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.DTYPE_CODE[q.dtype], B, Hq, Hkv, _HEAD_DIM, L, past_len, rows,
-        float(scale), _lib.ptr(out), _lib.stream_ptr()), "flash_prefill")
+        float(scale), _lib.ptr(out), _lib.ptr(workspace), workspace.numel() * workspace.element_size(),
+        _lib.stream_ptr()), "flash_prefill")
     return out

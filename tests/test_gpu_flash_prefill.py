@@ -33,6 +33,8 @@ def _case(B, Hq, Hkv, L, past, dtype, seed, extra_rows=0):
     (1, 4, 2, 1, 300, torch.bfloat16, 0),
     (1, 2, 2, 257, 31, torch.float16, 3),
     (1, 16, 2, 256, 2048, torch.bfloat16, 0),
+    (1, 16, 2, 64, 4100, torch.bfloat16, 0),   # short chunk over a deep prefix: key-range splits + merge
+    (1, 8, 2, 33, 3000, torch.float16, 7),
 ])
 def test_flash_prefill_matches_oracle(B, Hq, Hkv, L, past, dtype, extra):
     from moespresso_amd.runtime.qwen import kquant
@@ -100,6 +102,8 @@ def _q8_inputs(past, L, seed, sb_dtype=torch.float32, Hq=16, Hkv=2, B=1):
     (77, 33, torch.bfloat16, torch.bfloat16),
     (1024, 256, torch.float16, torch.float32),
     (31, 1, torch.float32, torch.float32),
+    (4133, 40, torch.float32, torch.float32),   # key-range splits over the quantised prefix
+    (6000, 256, torch.bfloat16, torch.float32),
 ])
 def test_sdpa_fa_prefill_q8_matches_oracle(past, L, sb_dtype, self_dtype):
     """Tolerance 1e-2 max-abs (8-bit KV bar) vs float64 attention over the dequantised prefix + chunk."""
