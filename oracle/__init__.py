@@ -29,4 +29,10 @@ would fail; "unpinned" = only self-consistency is available):
   q8 quantisers (affine g64)         parity unpinned (MLX mx.quantize edge rules not in the
                                      reference tree; own documented rule, round trip bounded)
   gqa decode / causal flash prefill  pinned  (float64 torch.softmax closed form)
+  indexer_q_qat_live                 tie rule pinned (the seven lattice midpoints, hand values) and
+                                     scale rule pinned on exact inputs; parity unpinned within an ulp
+                                     of a power of two (Metal log2/exp2 bits unknown; the reference
+                                     tests this kernel to 1e-5 only)
+  indexer_scores_tiled_live          pinned  (term-by-term float64 sum on half-rounded operands,
+                                     visibility against the closed form)
 """
