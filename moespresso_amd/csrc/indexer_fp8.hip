@@ -13,11 +13,20 @@
 
 namespace {
 
-// Two E4M3FN bytes (the low or high half of `w`) to two bf16 values packed in one register.
+// Two E4M3FN bytes (the low or high half of `w`) to two bf16 values packed in one register: one
+// conversion instruction (the scale operand is 1; every E4M3 value is exact in bf16).
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t fp8x2_to_bf16x2(uint32_t w, bool hi) {
-  f32x2_t f = hi ? __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true) : __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
-  // bf16 = top 16 bits of the float32 (exact: E4M3 carries 3 mantissa bits)
-  return __builtin_amdgcn_perm(__float_as_uint(f.y), __float_as_uint(f.x), 0x07060302u);
+  bf16x2_t r = hi ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true)
+                  : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// max(x, 0) on the bit pattern: a float with the sign bit set is a negative integer. One instruction,
+// where the float maximum first spends another one on quieting its operand.
+__device__ __forceinline__ float relu_bits(float x) {
+  const int v = __float_as_int(x);
+  return __int_as_float(v > 0 ? v : 0);
 }
 
 __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16_t* __restrict__ q,
@@ -101,9 +110,9 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
     }
     float sum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 16; i++) sum = fmaf(fmaxf(acc0[i], 0.0f), wl[0][i], sum);
+    for (int i = 0; i < 16; i++) sum = fmaf(relu_bits(acc0[i]), wl[0][i], sum);
 #pragma unroll
-    for (int i = 0; i < 16; i++) sum = fmaf(fmaxf(acc1[i], 0.0f), wl[1][i], sum);
+    for (int i = 0; i < 16; i++) sum = fmaf(relu_bits(acc1[i]), wl[1][i], sum);
     sum += __shfl_xor(sum, 32, MSPR_WAVE);
     if (g == 0 && row < n_rows) sb[row] = sum * ks;
   };

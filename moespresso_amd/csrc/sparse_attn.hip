@@ -85,7 +85,7 @@ struct SparseAttnArgs {
   int n_splits;
   int slots_per_split;
   int n_hblk;
-  float* ws_o;
+  uint16_t* ws_o;  // float16 partial rows, each normalised by its own range's denominator
   float* ws_ml;
   // output
   void* out;
@@ -639,15 +639,30 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     }
     return;
   }
-  // ---- partial results: registers go out in their native order (coalesced), stats per head
+  // ---- partial results: registers go out in their native order (coalesced), stats per head. A
+  // partial row is stored normalised by its own denominator, so it is a convex combination of V rows
+  // and fits float16 whenever V does; with bf16 V it saturates at the float16 range instead of
+  // overflowing. Its rounding (2^-11 relative) stays below the rounding of the final output.
   const int64_t part = ((int64_t)(seq * a.n_hblk + hb) * a.n_splits + sp);
-  float* wo = a.ws_o + (part * 4 + wave) * (int64_t)(8 * 16 * 64);
+  uint16_t* wo = a.ws_o + (part * 4 + wave) * (int64_t)(8 * 16 * 64);
+  const float inv_l = l_tot == 0.0f ? 0.0f : 1.0f / l_tot;
 #pragma unroll
   for (int mt = 0; mt < 8; mt++)
 #pragma unroll
-    for (int c = 0; c < 4; c++)
-      *reinterpret_cast<f32x4_t*>(wo + ((mt * 4 + c) * 64 + lane) * 4) =
-          f32x4_t{oacc[mt][4 * c], oacc[mt][4 * c + 1], oacc[mt][4 * c + 2], oacc[mt][4 * c + 3]};
+    for (int c = 0; c < 4; c += 2) {
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        float x = oacc[mt][4 * c + 2 * j] * inv_l, y = oacc[mt][4 * c + 2 * j + 1] * inv_l;
+        if constexpr (KDT == MSPR_BF16) {
+          x = __builtin_amdgcn_fmed3f(x, -65504.0f, 65504.0f);
+          y = __builtin_amdgcn_fmed3f(y, -65504.0f, 65504.0f);
+        }
+        w[j] = pack2<MSPR_F16>(x, y);
+      }
+      // registers 4c..4c+7 of this lane: 16 bytes, lane-contiguous
+      *reinterpret_cast<u32x4_t*>(wo + ((mt * 2 + c / 2) * 64 + lane) * 8) = u32x4_t{w[0], w[1], w[2], w[3]};
+    }
   if (dh == 0 && g == 0) {
     float* ml = a.ws_ml + (part * 64 + hg * 32 + n) * 2;
     ml[0] = m_run;
@@ -661,7 +676,7 @@ template <int ODT>
 __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int c = tid >> 6;  // accumulator quad: registers 4c..4c+3
+  const int c = tid >> 6;  // accumulator quad: registers 4c..4c+3 (half of a stored group of 8)
   const int mt = blockIdx.x & 7;
   const int wave = (blockIdx.x >> 3) & 3;
   const int bh = blockIdx.x >> 5;
@@ -677,7 +692,8 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   const float sink = load_sink_log2(a, head);
   const int64_t part0 = (int64_t)(seq * a.n_hblk + hb) * a.n_splits;
   const float* ml0 = a.ws_ml + (part0 * 64 + hg * 32 + n) * 2;
-  const float* wo0 = a.ws_o + (part0 * 4 + wave) * (int64_t)(8 * 16 * 64) + ((mt * 4 + c) * 64 + lane) * 4;
+  const uint16_t* wo0 =
+      a.ws_o + (part0 * 4 + wave) * (int64_t)(8 * 16 * 64) + ((mt * 2 + c / 2) * 64 + lane) * 8 + (c & 1) * 4;
   // One online pass in chunks of 16 ranges: the statistics and the partial rows of a chunk are all
   // requested at once, so a sequence split into up to 16 ranges costs one memory round trip.
   constexpr int kChunk = 16;
@@ -686,14 +702,14 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   f32x4_t o = {0.f, 0.f, 0.f, 0.f};
   for (int s0 = 0; s0 < a.n_splits; s0 += kChunk) {
     float mv[kChunk], lv[kChunk];
-    f32x4_t ov[kChunk];
+    f16x4_t ov[kChunk];
 #pragma unroll
     for (int j = 0; j < kChunk; j++) {
       const bool live = s0 + j < a.n_splits;
       const int64_t sj = live ? s0 + j : 0;
       mv[j] = ml0[sj * 128];
       lv[j] = ml0[sj * 128 + 1];
-      ov[j] = *reinterpret_cast<const f32x4_t*>(wo0 + sj * (int64_t)(4 * 8 * 16 * 64));
+      ov[j] = *reinterpret_cast<const f16x4_t*>(wo0 + sj * (int64_t)(4 * 8 * 16 * 64));
       if (!live) mv[j] = -__builtin_inff();
     }
     float m_new = m_run;
@@ -705,9 +721,9 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
     o = o * alpha;
 #pragma unroll
     for (int j = 0; j < kChunk; j++) {
-      const float w = fast_exp2(mv[j] - m_safe);
-      l += lv[j] * w;
-      o += ov[j] * w;
+      const float w = lv[j] * fast_exp2(mv[j] - m_safe);  // the stored row is already divided by lv[j]
+      l += w;
+      o += __builtin_convertvector(ov[j], f32x4_t) * w;
     }
     m_run = m_new;
   }
@@ -738,7 +754,7 @@ size_t workspace_bytes(int batch, int n_heads, int64_t n_keys) {
   int splits = choose_splits(batch * n_hblk, (int)n_keys);
   if (splits == 1) return 256;  // one key range per sequence: stored directly, no partials
   size_t parts = (size_t)batch * n_hblk * splits;
-  return parts * (4 * 8 * 16 * 64 * sizeof(float)) + parts * 64 * 2 * sizeof(float) + 256;
+  return parts * (4 * 8 * 16 * 64 * sizeof(uint16_t)) + parts * 64 * 2 * sizeof(float) + 256;
 }
 
 template <int KDT, int DK, int QDT, bool ROPE>
@@ -786,8 +802,8 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
                need, workspace_bytes_given);
   MSPR_REQUIRE(mspr_aligned(workspace, 16), "sparse attention: workspace must be 16-byte aligned");
   size_t parts = (size_t)a.batch * a.n_hblk * a.n_splits;
-  a.ws_o = reinterpret_cast<float*>(workspace);
-  a.ws_ml = a.ws_o + parts * (4 * 8 * 16 * 64);
+  a.ws_o = reinterpret_cast<uint16_t*>(workspace);
+  a.ws_ml = reinterpret_cast<float*>(a.ws_o + parts * (4 * 8 * 16 * 64));
 #ifdef MSPR_SPARSE_TRACE
   a.trace = g_trace_buf;
 #endif
