@@ -1,17 +1,21 @@
-// Deterministic top-k over float32 score rows: MSB radix select on monotone uint32 keys (four
-// 8-bit digits), then ordered emission (rows strictly above the k-th key in ascending row order,
-// then the lowest-index rows tied with it).
+// Deterministic top-k over float32 score rows: select on monotone uint32 keys, then ordered emission
+// (rows strictly above the k-th key in ascending row order, then the lowest-index rows tied with it).
 //
-// One 1024-thread workgroup per score row. For rows of up to CACHE*1024 scores every thread keeps
-// its keys in registers (striped ownership: thread t owns rows t, t+1024, ...), so HBM/L2 is read
-// once; longer rows re-read global memory each pass.
-//
-// Histograms: 256 bins x 64 copies in LDS, copy = lane id, laid out [bin][copy]. Every lane of an
-// LDS atomic then hits its own bank whatever the digit distribution is (scores of one row usually
-// share their top byte, which would serialise a single shared counter 64-fold).
-//
-// After the first two digits the keys that still match the 16-bit prefix are usually a handful;
-// they are compacted into an LDS list and the last two digits run on that list only.
+// One 1024-thread workgroup per score row. Rows of up to 32768 scores are read once and kept in
+// registers, every thread owning a block of consecutive rows. Two ways to the k-th key:
+//  * pivot path: a 1024-row sample gives a 16-bit key prefix safely below the k-th key, the rows at
+//    or above it (a few thousand) are compacted in row order and three small digit passes plus the
+//    emission run on that list. The kernel checks exactly that the list contains the k-th key; the
+//    sample decides how long the call takes, never what it returns.
+//  * full passes (also the fallback of the pivot path): MSB radix select with four 8-bit digits over
+//    all keys. Histograms are 256 bins x 64 copies in LDS, copy = lane id, laid out [bin][copy], so
+//    every lane of an LDS atomic hits its own bank whatever the digit distribution is (scores of one
+//    row usually share their top byte, which would serialise a single shared counter 64-fold). After
+//    two digits the keys that still match the prefix are usually a handful; they are compacted into
+//    an LDS list and the last two digits run on that list only.
+// Longer rows use the striped kernel, which re-reads global memory each pass.
+#include <cmath>
+
 #include "common.h"
 #include "profile.h"
 
@@ -37,6 +41,8 @@ constexpr int kThreads = 1024;
 constexpr int kWaves = kThreads / 64;
 constexpr int kCopies = 64;
 constexpr int kListCap = 2048;
+constexpr int kFastPer = 6;                     // survivor-list entries per thread on the pivot path
+constexpr int kFastCap = kFastPer * kThreads;   // survivor-list capacity
 
 struct SelectState {
   uint32_t prefix;
@@ -324,6 +330,26 @@ __device__ __forceinline__ uint32_t wave_prefix_sum(uint32_t x) {
   return (uint32_t)v;
 }
 
+// mask = 2 mask + bit
+__device__ __forceinline__ uint32_t shift_in(uint32_t mask, bool bit) { return (mask << 1) | (bit ? 1u : 0u); }
+
+// One histogram vote per lane. Up to four rounds first count all lanes that share the bin of the
+// lowest voting lane with a single atomic (digits near the top of the key are shared by most rows,
+// which would serialise one atomic per lane on the same counter); what is left votes directly.
+__device__ __forceinline__ void wave_hist_add(uint32_t* h, int bin, int lane) {
+#pragma unroll
+  for (int round = 0; round < 4; round++) {
+    const uint64_t voters = __ballot(bin >= 0);
+    if (voters == 0ull) break;
+    const int first = (int)__builtin_ctzll(voters);
+    const int d = __builtin_amdgcn_readlane(bin, first);
+    const uint64_t same = __ballot(bin == d);
+    if (lane == first) atomicAdd(&h[d], (uint32_t)__popcll(same));
+    if (bin == d) bin = -1;
+  }
+  if (bin >= 0) atomicAdd(&h[bin], 1u);
+}
+
 __device__ __forceinline__ Pick pick_bucket(const uint32_t* totals, uint32_t need, int lane) {
   // lane l looks at digits 255-4l .. 252-4l, so a prefix sum over lanes counts keys from the top digit down
   uint32_t t[4];
@@ -373,30 +399,37 @@ __device__ __forceinline__ Pick pick_bucket(const uint32_t* totals, uint32_t nee
 template <int C>
 __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __restrict__ scores_all,
                                                                  int64_t score_stride, int n_rows, int topk,
-                                                                 int32_t* __restrict__ sel_all) {
+                                                                 int sample_rank, int32_t* __restrict__ sel_all) {
   // The staging area for the load (C*1024 keys) is reused for the histogram copies afterwards.
   constexpr int kStageWords = C * kThreads > 256 * kCopies ? C * kThreads : 256 * kCopies;
   __shared__ __attribute__((aligned(16))) uint32_t stage[kStageWords];
   uint32_t* hist = stage;                   // [bin][copy]
   __shared__ uint32_t totals[256];
   __shared__ uint32_t small_hist[2][256];   // digits 2 and 3 on the compacted list
-  __shared__ uint32_t list[kListCap];
+  // survivor rows of the pivot path (16-bit row numbers), or the compacted keys of the full passes
+  __shared__ __attribute__((aligned(16))) uint32_t list_words[kFastCap / 2 > kListCap ? kFastCap / 2 : kListCap];
+  uint32_t* list = list_words;
+  uint16_t* fast_rows = reinterpret_cast<uint16_t*>(list_words);
   __shared__ uint32_t list_n;
   __shared__ uint32_t wave_tot[kWaves];
+  __shared__ uint32_t fhist[5][256];        // pivot path: two sample digits, three digits on the survivor list
+  __shared__ Pick pick_box[5];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const float* scores = scores_all + (int64_t)blockIdx.x * score_stride;
   int32_t* sel = sel_all + (int64_t)blockIdx.x * topk;
+  if (sample_rank > 0)
+    for (int i = tid; i < 5 * 256; i += kThreads) (&fhist[0][0])[i] = 0u;  // ordered by the barriers of the load
 
   TOPK_STAMP(0);
   // Load with lane-contiguous 16-byte reads (a wave reads 1 KB at a time), then hand every thread its
   // C consecutive rows through LDS. The 16-byte pieces of a thread's C/4-piece block are XOR-permuted
   // by the thread index so that neither the writes nor the reads pile up on a few banks.
   uint32_t kreg[C];
+  constexpr int kPieces = C / 4;  // 16-byte pieces per thread
   {
-    constexpr int kPieces = C / 4;  // 16-byte pieces per thread
     const bool vec_ok = (reinterpret_cast<uintptr_t>(scores) & 15u) == 0u && n_rows >= 4;  // uniform
     // all vector loads first, unconditionally (a piece that crosses the end of the row re-reads the
     // last whole piece and is patched element by element below)
@@ -430,8 +463,133 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
 #pragma unroll
       for (int e = 0; e < 4; e++) kreg[4 * j + e] = keys[e];
     }
-    __syncthreads();
   }
+  TOPK_STAMP(1);
+
+  // ---- pivot path. Every thread's first row is a sample of the (padded) row set; the 16-bit key
+  // prefix at rank `sample_rank` of the sample sits, with a wide margin, below the k-th key of the
+  // whole row, so the rows at or above it ("survivors", a few thousand) contain the answer. They are
+  // compacted in row order and the exact select and the emission run on that list only. Whether the
+  // pivot was good is checked exactly (survivors >= k, within the list capacity, k-th key less than
+  // 255 prefixes above the pivot); if not, the full radix passes below take over, so the result never
+  // depends on the sample. The keys stay in the staging area, which this path does not overwrite.
+  // one wave works out the digit, the others wait for it: with 16 waves on 4 SIMDs a computation that
+  // every wave repeats costs four times its instruction count, a barrier costs less (a slot per use,
+  // so no slot is rewritten while a slow wave may still read it)
+  auto shared_pick = [&](const uint32_t* h, uint32_t want, int slot) -> Pick {
+    if (wave == 0) {
+      const Pick p = pick_bucket(h, want, lane);
+      if (lane == 0) pick_box[slot] = p;
+    }
+    __syncthreads();
+    return pick_box[slot];
+  };
+  if (sample_rank > 0) {
+    const uint32_t skey = kreg[0];
+    wave_hist_add(fhist[0], (int)(skey >> 24), lane);  // the top byte is shared by most rows: vote per wave
+    __syncthreads();
+    const Pick s0 = shared_pick(fhist[0], (uint32_t)sample_rank, 0);
+    if ((skey >> 24) == s0.digit) atomicAdd(&fhist[1][(skey >> 16) & 0xFFu], 1u);
+    __syncthreads();
+    const Pick s1 = shared_pick(fhist[1], s0.need, 1);
+    const uint32_t pivot16 = (s0.digit << 8) | s1.digit;
+    const uint32_t pivot = pivot16 << 16;
+    TOPK_STAMP(2);
+
+    uint32_t smask = 0u;
+#pragma unroll
+    for (int i = C - 1; i >= 0; i--) smask = shift_in(smask, kreg[i] >= pivot);
+    const uint32_t cnt = (uint32_t)__popc(smask);
+    const uint32_t sincl = wave_prefix_sum(cnt);
+    if (lane == 63) wave_tot[wave] = sincl;
+    __syncthreads();
+    uint32_t sbase = 0u, total = 0u;
+#pragma unroll
+    for (int w = 0; w < kWaves; w++) {
+      const uint32_t wt = wave_tot[w];
+      sbase += w < wave ? wt : 0u;
+      total += wt;
+    }
+    TOPK_STAMP(3);
+    if (total >= (uint32_t)topk && total <= (uint32_t)kFastCap) {  // the same for every thread
+      uint32_t pos = sbase + sincl - cnt;
+      while (smask) {
+        const int i = __builtin_ctz(smask);
+        smask &= smask - 1u;
+        fast_rows[pos++] = (uint16_t)(C * tid + i);
+      }
+      __syncthreads();
+      TOPK_STAMP(4);
+      // thread t takes the list entries [t E, t E + E): consecutive, so the emission order is again a
+      // matter of one block scan
+      const uint32_t per = (total + kThreads - 1) / kThreads;  // 1 .. kFastPer
+      uint32_t lk[kFastPer], lr[kFastPer];
+      uint32_t lvalid = 0u;
+#pragma unroll
+      for (int j = 0; j < kFastPer; j++) {
+        const uint32_t idx = (uint32_t)tid * per + j;
+        const bool ok = (uint32_t)j < per && idx < total;
+        const uint32_t row = fast_rows[ok ? idx : 0u];
+        const uint32_t owner = row / C, piece = (row % C) >> 2, e = row & 3u;
+        lr[j] = row;
+        lk[j] = stage[owner * C + 4 * (piece ^ (owner & (kPieces - 1))) + e];
+        lvalid |= (ok ? 1u : 0u) << j;
+      }
+      // digit A: distance of the 16-bit prefix from the pivot's, everything 255 or more prefixes up in
+      // one bin; digits B and C: the low 16 bits
+      uint32_t* hA = fhist[2];
+#pragma unroll
+      for (int j = 0; j < kFastPer; j++) {
+        const uint32_t d = (lk[j] >> 16) - pivot16;
+        if ((lvalid >> j) & 1u) atomicAdd(&hA[d < 255u ? d : 255u], 1u);
+      }
+      __syncthreads();
+      const Pick pa = shared_pick(hA, (uint32_t)topk, 2);
+      if (pa.digit < 255u) {  // the same for every thread
+        uint32_t fprefix = (pivot16 + pa.digit) << 16, fneed = pa.need;
+#pragma unroll
+        for (int pass = 2; pass < 4; pass++) {
+          const uint32_t shift = 24u - 8u * pass;
+          const uint32_t mask_hi = 0xFFFFFFFFu << (shift + 8u);
+          uint32_t* h = fhist[1 + pass];
+#pragma unroll
+          for (int j = 0; j < kFastPer; j++)
+            if (((lvalid >> j) & 1u) && (lk[j] & mask_hi) == fprefix) atomicAdd(&h[(lk[j] >> shift) & 0xFFu], 1u);
+          __syncthreads();
+          const Pick pk = shared_pick(h, fneed, 1 + pass);
+          fprefix |= pk.digit << shift;
+          fneed = pk.need;
+        }
+        TOPK_STAMP(14);
+        const uint32_t n_above_f = (uint32_t)topk - fneed;
+        uint32_t am = 0u, tm = 0u;
+#pragma unroll
+        for (int j = 0; j < kFastPer; j++) {
+          const bool ok = (lvalid >> j) & 1u;
+          am |= (ok && lk[j] > fprefix ? 1u : 0u) << j;
+          tm |= (ok && lk[j] == fprefix ? 1u : 0u) << j;
+        }
+        const uint32_t mine_f = (uint32_t)__popc(am) | ((uint32_t)__popc(tm) << 16);
+        const uint32_t incl_f = wave_prefix_sum(mine_f);
+        if (lane == 63) wave_tot[wave] = incl_f;  // its earlier contents were consumed before the barriers above
+        __syncthreads();
+        uint32_t base_f = 0u;
+        for (int w = 0; w < wave; w++) base_f += wave_tot[w];
+        const uint32_t excl_f = base_f + incl_f - mine_f;
+        uint32_t slot_f = excl_f & 0xFFFFu;
+        uint32_t rank_f = excl_f >> 16;
+#pragma unroll
+        for (int j = 0; j < kFastPer; j++) {
+          if ((am >> j) & 1u) sel[slot_f++] = (int32_t)lr[j];
+          else if (((tm >> j) & 1u) && rank_f < fneed) sel[n_above_f + rank_f++] = (int32_t)lr[j];
+        }
+        TOPK_STAMP(17);
+        return;
+      }
+    }
+  }
+  __syncthreads();  // the staging area and wave_tot have been read by every thread; the full passes reuse them
+
   {
     u32x4_t* h4 = reinterpret_cast<u32x4_t*>(hist);
     for (int i = tid; i < 256 * kCopies / 4; i += kThreads) h4[i] = u32x4_t{0u, 0u, 0u, 0u};
@@ -439,7 +597,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
     if (tid == 0) list_n = 0u;
   }
   __syncthreads();
-  TOPK_STAMP(1);
 
   uint32_t prefix = 0u, need = (uint32_t)topk, live = (uint32_t)(C * kThreads);
 
@@ -548,14 +705,29 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
   TOPK_STAMP(17);
 }
 
+// Rank, inside the 1024-row sample, of the pivot of the pivot path; 0 switches the path off. With k of
+// the C*1024 (padded) rows wanted, k/C sample rows are expected above the k-th key; the rank adds 4.5
+// standard deviations so that the survivors almost always include it, and the path is used only where
+// the survivors then almost always (6 more deviations) fit the list. A miss on either side costs time,
+// not correctness: the kernel checks the survivor count and falls back to the full passes.
+int pivot_sample_rank(int c, int topk) {
+  const double expect = (double)topk / c;
+  const double rank = std::ceil(expect + 4.5 * std::sqrt(expect) + 2.0);
+  const double worst = rank * c + 6.0 * c * std::sqrt(rank);
+  if (rank > 512.0 || worst > (double)kFastCap) return 0;
+  return (int)rank;
+}
+
 }  // namespace
 
 int mspr_launch_topk(const float* scores, int64_t score_stride, int batch, int64_t n_rows, int topk, int32_t* sel,
                      hipStream_t st) {
   dim3 grid((unsigned)batch), block(kThreads);
   MsprProfScope prof(MSPR_K_TOPK, st);
-  if (n_rows <= 8 * 1024) topk_blocked_kernel<8><<<grid, block, 0, st>>>(scores, score_stride, (int)n_rows, topk, sel);
-  else if (n_rows <= 32 * 1024) topk_blocked_kernel<32><<<grid, block, 0, st>>>(scores, score_stride, (int)n_rows, topk, sel);
+  if (n_rows <= 8 * 1024)
+    topk_blocked_kernel<8><<<grid, block, 0, st>>>(scores, score_stride, (int)n_rows, topk, pivot_sample_rank(8, topk), sel);
+  else if (n_rows <= 32 * 1024)
+    topk_blocked_kernel<32><<<grid, block, 0, st>>>(scores, score_stride, (int)n_rows, topk, pivot_sample_rank(32, topk), sel);
   else topk_select_kernel<0><<<grid, block, 0, st>>>(scores, score_stride, n_rows, topk, sel);
   MSPR_CHECK_LAUNCH("topk_select");
   return MSPR_OK;

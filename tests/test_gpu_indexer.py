@@ -313,6 +313,32 @@ def test_topk_select_bitexact(shape_k):
             np.testing.assert_array_equal(g2[b], ds4.radix_select_topk(rows[b], k))
 
 
+@pytest.mark.parametrize("n_k", [(32768, 2048), (32768, 512), (20000, 2048), (8192, 2048), (8192, 64), (3000, 1)])
+def test_topk_select_sample_misleads(n_k):
+    """The kernel guesses a pivot from every C-th row (C = 8 up to 8192 rows, 32 up to 32768) and must
+    fall back to the full select when the guess is bad: rows whose sampled positions are all small, all
+    large, or all equal must still give the exact answer."""
+    n, k = n_k
+    c = 8 if n <= 8192 else 32
+    rng = np.random.default_rng(n + k)
+    base = rng.standard_normal((4, n)).astype(np.float32)
+    lo = base.copy()
+    lo[:, ::c] = -50.0 - rng.random((4, len(range(0, n, c)))).astype(np.float32)   # pivot far too low
+    hi = base.copy()
+    hi[:, ::c] = 50.0 + rng.random((4, len(range(0, n, c)))).astype(np.float32)    # pivot far too high
+    eq = base.copy()
+    eq[:, ::c] = 0.25                                                              # one value in the sample
+    few = np.zeros((4, n), dtype=np.float32)                                       # k-th key inside a huge tie
+    few[:, rng.integers(0, n, max(1, k // 2))] = 1.0
+    edge = base.copy()                                                             # exactly k rows above the rest
+    edge[:, :] = -1.0
+    edge[:, rng.choice(n, k, replace=False)] = rng.random(k).astype(np.float32) + 1.0
+    for s in (lo, hi, eq, few, edge):
+        got = isk.topk_select(to_dev(s), k).cpu().numpy()
+        for b in range(s.shape[0]):
+            np.testing.assert_array_equal(got[b], ds4.radix_select_topk(s[b], k))
+
+
 def test_validation_messages_match_reference():
     # reference :125-133, :211-238, :752-776 (rejections happen before any device work)
     z = torch.zeros
