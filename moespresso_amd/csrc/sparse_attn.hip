@@ -5,13 +5,14 @@
 // a pool by index. K is the whole row (512 or 576 wide), V its first 512 columns.
 //
 // Work split: a workgroup owns (batch, 64-head block, slot range) and streams 32-slot tiles.
-// Each K row is read from HBM once and staged row-major in LDS (double buffered). The four waves
-// are (head group hg of 32 heads) x (half dh): for S^T = K.Q^T a wave contracts its half of the
-// row width and the two halves are summed through LDS; for O^T = V^T.P^T it owns 256 of the 512
-// output columns. V^T operands come out of the same row-major tile through the LDS transpose
-// read, so no second copy of the tile exists. Partial (m, l, O) per slot range are merged by a
-// second kernel (log-sum-exp), which also applies the sink, the normalisation, the output cast
-// and the optional inverse rope.
+// Each K row is read from HBM once and staged row-major in LDS (ring of three tiles, filled by
+// asynchronous global->LDS copies). The eight waves are (head group hg of 32 heads) x (quarter dh):
+// for S^T = K.Q^T a wave contracts its quarter of the row width and the four quarters are summed
+// through LDS; for O^T = V^T.P^T it owns 128 of the 512 output columns. Two waves share a SIMD: one
+// wave alone can issue a 32x32x16 MFMA only every other slot of the matrix pipe. V^T operands come
+// out of the same row-major tile through the LDS transpose read, so no second copy of the tile
+// exists. Partial (m, l, O) per slot range are merged by a second kernel (log-sum-exp), which also
+// applies the sink, the normalisation, the output cast and the optional inverse rope.
 //
 // MFMA shapes: v_mfma_f32_32x32x16_{f16,bf16}. Accumulator layout (lane l, register i):
 // column = l % 32, row = 8*(i/4) + 4*(l/32) + i%4. In S^T the column is the head and the row the
@@ -37,7 +38,8 @@ namespace {
 
 constexpr int kTile = 32;
 constexpr int kDV = 512;
-constexpr int kThreads = 256;
+constexpr int kThreads = 512;  // split kernel: eight waves, two per SIMD
+constexpr int kWaves = kThreads / 64;
 
 struct SparseAttnArgs {
   // query
@@ -214,12 +216,13 @@ struct Geometry {
   static constexpr int kPitch = kSlots * 16;       // bytes
   static constexpr int kTileSlots = kTile * kSlots;
   static constexpr int kInstr = (kTileSlots + 63) / 64;   // wave-wide 1 KB loads per tile
-  static constexpr int kPerThread = (kInstr + 3) / 4;     // loads per thread per tile (wave 0 issues the odd one)
+  static constexpr int kPerThread = (kInstr + kWaves - 1) / kWaves;  // loads per thread per tile
+  static constexpr int kLastWaves = kInstr - kWaves * (kPerThread - 1);  // waves that issue the last of them
   static constexpr int kTileBytes = kInstr * 1024;
-  static constexpr int kHalf = DK / 2;             // contraction columns per dh wave
-  static constexpr int kSteps = kHalf / 16;        // MFMA k-steps per dh wave
+  static constexpr int kPart = DK / 4;             // contraction columns per dh wave
+  static constexpr int kSteps = kPart / 16;        // MFMA k-steps per dh wave
   static constexpr int kBufs = 3;                  // tile ring: one in use, two in flight
-  static constexpr int kSxBytes = 4 * 16 * 64 * 4; // 4 waves x 16 floats x 64 lanes
+  static constexpr int kSxBytes = 4 * 16 * 64 * 4; // 4 waves x 16 floats x 64 lanes (one head group)
   static constexpr int kMaxIds = 1024;             // gathered slots per workgroup
   static constexpr int kOffSx = kBufs * kTileBytes;
   static constexpr int kMaxTiles = kMaxIds / kTile; // tiles per workgroup (slots_per_split <= kMaxIds)
@@ -228,7 +231,8 @@ struct Geometry {
   static constexpr int kOffRope = kOffVmask + kMaxTiles * 4;
   static constexpr int kOffStop = kOffRope + 64 * 4;
   static constexpr int kLdsBytes = kOffStop + 16;
-  static_assert(kInstr % 4 == 1, "wave 0 issues exactly one load more than the other waves");
+  static_assert(kPart % 16 == 0, "a wave's share of the row width is a whole number of MFMA k-steps");
+  static_assert(kLastWaves >= 1 && kLastWaves <= kWaves, "the last round of tile loads is issued by the first waves");
 };
 
 template <int KDT, int DK, int QDT, bool ROPE>
@@ -236,7 +240,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   using G = Geometry<DK>;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   unsigned char* kbuf = lds;                                                   // [kBufs][kTileBytes]
-  float* sx = reinterpret_cast<float*>(lds + G::kOffSx);                       // [2][4][16*64]
+  float* sx = reinterpret_cast<float*>(lds + G::kOffSx);                       // [8 waves][16*64]
   uint64_t* rowptr = reinterpret_cast<uint64_t*>(lds + G::kOffRowPtr);         // [kMaxIds]
   uint32_t* vmask = reinterpret_cast<uint32_t*>(lds + G::kOffVmask);           // [kMaxTiles]
   float* rope_c = reinterpret_cast<float*>(lds + G::kOffRope);
@@ -246,8 +250,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int hg = wave >> 1;
-  const int dh = wave & 1;
+  const int hg = wave >> 2;  // head group of 32 heads
+  const int dh = wave & 3;   // quarter of the row width (S^T) and of the output columns (O^T)
   const int n = lane & 31;  // MFMA column: head (S^T, O^T); MFMA row for A operands
   const int g = lane >> 5;
 
@@ -291,12 +295,12 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   const int32_t* idx_b = a.idx + (int64_t)seq * a.idx_batch_stride;
 
   MSPR_STAMP(0);
-  // ---- query operand: lane (n = head, g) holds q[head][dh*kHalf + 16ks + 8g .. +7]; its loads go out
+  // ---- query operand: lane (n = head, g) holds q[head][dh*kPart + 16ks + 8g .. +7]; its loads go out
   //      right behind the id loads below and are back by the time the row pointer table is built
   const int head = hb * 64 + hg * 32 + n;
   const bool q_live = head < a.n_heads;
   const int64_t qoff = (int64_t)b * a.q_batch_stride + (int64_t)t * a.q_token_stride +
-                       (int64_t)(q_live ? head : 0) * a.q_head_stride + dh * G::kHalf + 8 * g;
+                       (int64_t)(q_live ? head : 0) * a.q_head_stride + dh * G::kPart + 8 * g;
   u32x4_t qf[G::kSteps];
   f32x4_t qraw32[QDT == MSPR_F32 ? G::kSteps : 1][2];
   // The gathered ids of this thread's slots are requested before anything else: ids -> row pointers ->
@@ -345,7 +349,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   uint32_t pk[G::kPerThread];
 #pragma unroll
   for (int j = 0; j < G::kPerThread; j++) {
-    const int P = tid + 256 * j;
+    const int P = tid + kThreads * j;
     const int row = P / G::kSlots, chunk = P % G::kSlots;
     pk[j] = (P < G::kTileSlots && chunk != G::kSlots - 1) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
   }
@@ -406,7 +410,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, kbuf + (tile % G::kBufs) * G::kTileBytes + wave * 1024));
   };
   auto issue_one = [&](const uint64_t (&src)[G::kPerThread], uint32_t dst_lds, int j) {
-    if (j < G::kPerThread - 1 || wave == 0) async_load_16(src[j], dst_lds + j * 4096);
+    if (j < G::kPerThread - 1 || wave < G::kLastWaves) async_load_16(src[j], dst_lds + j * (kWaves * 1024));
   };
   auto issue_tile = [&](int tile) {
     uint64_t src[G::kPerThread];
@@ -418,6 +422,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 
   MSPR_STAMP(1);
   __syncthreads();  // row pointer table visible
+  MSPR_STAMP(61);
   // The query loads (issued long ago) must be complete before the first asynchronous tile load goes
   // out: a wait left for their first use would otherwise also wait for (drain) the tile loads behind them.
   if constexpr (QDT == MSPR_F32) {
@@ -427,6 +432,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 #pragma unroll
     for (int ks = 0; ks < G::kSteps; ks++) asm volatile("" : "+v"(qf[ks]));
   }
+  MSPR_STAMP(60);
   if (n_tiles > 0) issue_tile(0);
   if (n_tiles > 1) issue_tile(1);
   MSPR_STAMP(2);
@@ -451,7 +457,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
           v[2 * j + 1] = unpack_hi<KDT>(qf[ks][j]);
         }
       }
-      const int d0 = dh * G::kHalf + 16 * ks + 8 * g;
+      const int d0 = dh * G::kPart + 16 * ks + 8 * g;
       if (ROPE && d0 >= DK - 64) {
         // partial rope on interleaved pairs with every product and sum rounded to the element type
 #pragma unroll
@@ -472,9 +478,9 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   }
   MSPR_STAMP(3);
 
-  f32x16_t oacc[8];
+  f32x16_t oacc[4];
 #pragma unroll
-  for (int mt = 0; mt < 8; mt++) oacc[mt] = f32x16_t{0};
+  for (int mt = 0; mt < 4; mt++) oacc[mt] = f32x16_t{0};
   // m_run is a lazily updated reference maximum: it only moves when a tile's maximum exceeds it by
   // more than kGrow (log2 units), so the 128 accumulator registers are rescaled a few times per kernel
   // instead of once per tile.
@@ -482,22 +488,15 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   float l_run = 0.0f;
 
   // per-lane LDS offsets
-  const int a_row_off = n * G::kPitch + (dh * G::kHalf + 8 * g) * 2;  // QK^T A operand
+  const int a_row_off = n * G::kPitch + (dh * G::kPart + 8 * g) * 2;  // QK^T A operand
   const int tr_s = lane & 15;
-  const int tr_off = (4 * g + (tr_s >> 2)) * G::kPitch + (dh * 256 + 16 * ((lane >> 4) & 1) + 4 * (tr_s & 3)) * 2;
+  const int tr_off = (4 * g + (tr_s >> 2)) * G::kPitch + (dh * 128 + 16 * ((lane >> 4) & 1) + 4 * (tr_s & 3)) * 2;
 
   for (int t = 0; t < n_tiles; t++) {
-    // tile t has landed once this wave's loads of it are done and every wave got here
-    if (t + 1 < n_tiles) {
-      if (wave == 0) wait_vm_and_barrier<G::kPerThread>();
-      else wait_vm_and_barrier<G::kPerThread - 1>();
-    } else {
-      wait_vm_and_barrier<0>();
-    }
-    MSPR_STAMP(4 + 6 * t);
-    // tile t+2 goes into the ring buffer of tile t-1, which every wave has left; its copies are issued
-    // between the matrix-core instructions below, so that the time a copy waits for the address unit
-    // is covered by MFMAs already in flight
+    // tile t+2 goes into the ring buffer of tile t-1, which every wave has left after the barrier
+    // below; its copies are issued between the matrix-core instructions of this tile, so that the time
+    // a copy waits for the address unit is covered by MFMAs already in flight. The source addresses
+    // (reads of the static row pointer table) are worked out before the wait, in its shadow.
     const bool more = t + 2 < n_tiles;  // workgroup-uniform
     uint64_t nsrc[G::kPerThread];
     uint32_t ndst = 0;
@@ -505,15 +504,26 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       tile_sources(t + 2, nsrc);
       ndst = tile_lds_base(t + 2);
     }
+    // tile t has landed once this wave's loads of it are done and every wave got here
+    if (t + 1 < n_tiles) {
+      if (wave < G::kLastWaves) wait_vm_and_barrier<G::kPerThread>();
+      else wait_vm_and_barrier<G::kPerThread - 1>();
+    } else {
+      wait_vm_and_barrier<0>();
+    }
+    MSPR_STAMP(4 + 6 * t);
     const int buf = t % G::kBufs;
     const unsigned char* kt = kbuf + buf * G::kTileBytes;
     const uint32_t mask_all = vmask[t];
 
     MSPR_STAMP(5 + 6 * t);
     // S^T partial over this wave's half of the row width
+    // (two accumulators, even and odd k-steps: a wave is alone on its SIMD, so a single chain of
+    // dependent MFMAs would run at the instruction's latency instead of its issue rate)
     f32x16_t sacc = {0};
     {
-      constexpr int kAhead = 6;  // LDS reads in flight in front of the dependent MFMA chain
+      f32x16_t sodd = {0};
+      constexpr int kAhead = 6;  // LDS reads in flight in front of the MFMA chains
       u32x4_t af[kAhead];
 #pragma unroll
       for (int ks = 0; ks < kAhead; ks++) af[ks] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + ks * 32);
@@ -522,18 +532,23 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         u32x4_t cur = af[ks % kAhead];
         if (ks + kAhead < G::kSteps)
           af[ks % kAhead] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + (ks + kAhead) * 32);
-        sacc = mfma32<KDT>(cur, qf[ks], sacc);
+        if (ks & 1) sodd = mfma32<KDT>(cur, qf[ks], sodd);
+        else sacc = mfma32<KDT>(cur, qf[ks], sacc);
         if (more && (ks & 1) == 0 && ks / 2 < G::kPerThread) {
           issue_one(nsrc, ndst, ks / 2);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      sacc = sacc + sodd;
     }
     if (more) {
 #pragma unroll
       for (int j = (G::kSteps + 1) / 2; j < G::kPerThread; j++) issue_one(nsrc, ndst, j);
     }
-    float* sxw = sx + ((t & 1) * 4 + wave) * (16 * 64);
+    // the four partial S^T of a head group meet in LDS; every wave adds them in the same order, so the
+    // four waves hold bit-identical scores (one buffer is enough: the barrier at the top of the loop
+    // separates these reads from the next tile's writes)
+    float* sxw = sx + wave * (16 * 64);
 #pragma unroll
     for (int c = 0; c < 4; c++)
       *reinterpret_cast<f32x4_t*>(sxw + (c * 64 + lane) * 4) =
@@ -541,14 +556,22 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     MSPR_STAMP(6 + 6 * t);
     lds_barrier();
     MSPR_STAMP(7 + 6 * t);
-    const float* sxp = sx + ((t & 1) * 4 + (wave ^ 1)) * (16 * 64);
+    {
+      const float* sxp = sx + (hg * 4) * (16 * 64);
+      f32x4_t part[4][4];
 #pragma unroll
-    for (int c = 0; c < 4; c++) {
-      f32x4_t o = *reinterpret_cast<const f32x4_t*>(sxp + (c * 64 + lane) * 4);
-      sacc[4 * c] += o.x;
-      sacc[4 * c + 1] += o.y;
-      sacc[4 * c + 2] += o.z;
-      sacc[4 * c + 3] += o.w;
+      for (int d = 0; d < 4; d++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          part[d][c] = *reinterpret_cast<const f32x4_t*>(sxp + d * (16 * 64) + (c * 64 + lane) * 4);
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const f32x4_t o = ((part[0][c] + part[1][c]) + part[2][c]) + part[3][c];
+        sacc[4 * c] = o.x;
+        sacc[4 * c + 1] = o.y;
+        sacc[4 * c + 2] = o.z;
+        sacc[4 * c + 3] = o.w;
+      }
     }
 
     // online softmax in the log2 domain; key of register i is 8*(i/4) + 4g + i%4
@@ -580,7 +603,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       m_run = m_new;
       if (!fresh) {
 #pragma unroll
-        for (int mt = 0; mt < 8; mt++) oacc[mt] = oacc[mt] * alpha;
+        for (int mt = 0; mt < 4; mt++) oacc[mt] = oacc[mt] * alpha;
       }
     }
     const float m_safe = m_run == -__builtin_inff() ? 0.0f : m_run;
@@ -599,10 +622,11 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 
     MSPR_STAMP(8 + 6 * t);
     // O^T += V^T . P^T ; V^T operands through the LDS transpose read of the row-major tile
+    // (k-step outer, output tile inner: consecutive MFMAs never share an accumulator)
 #pragma unroll
-    for (int mt = 0; mt < 8; mt++) {
+    for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
+      for (int mt = 0; mt < 4; mt++) {
         const unsigned char* base = kt + tr_off + (16 * ks) * G::kPitch + mt * 64;
         s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base));
         s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base + 8 * G::kPitch));
@@ -626,12 +650,12 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       const int64_t obase = (int64_t)b * a.out_batch_stride + (int64_t)t * a.out_token_stride +
                             (int64_t)head * a.out_head_stride;
 #pragma unroll
-      for (int mt = 0; mt < 8; mt++)
+      for (int mt = 0; mt < 4; mt++)
 #pragma unroll
         for (int c = 0; c < 4; c++) {
           const float r[4] = {oacc[mt][4 * c] * f, oacc[mt][4 * c + 1] * f, oacc[mt][4 * c + 2] * f,
                               oacc[mt][4 * c + 3] * f};
-          const int dim0 = dh * 256 + 32 * mt + 8 * c + 4 * g;
+          const int dim0 = dh * 128 + 32 * mt + 8 * c + 4 * g;
           if (a.out_dtype == MSPR_F32) emit_output<MSPR_F32>(a, r, obase + dim0, dim0);
           else if (a.out_dtype == MSPR_BF16) emit_output<MSPR_BF16>(a, r, obase + dim0, dim0);
           else emit_output<MSPR_F16>(a, r, obase + dim0, dim0);
@@ -644,10 +668,10 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   // and fits float16 whenever V does; with bf16 V it saturates at the float16 range instead of
   // overflowing. Its rounding (2^-11 relative) stays below the rounding of the final output.
   const int64_t part = ((int64_t)(seq * a.n_hblk + hb) * a.n_splits + sp);
-  uint16_t* wo = a.ws_o + (part * 4 + wave) * (int64_t)(8 * 16 * 64);
+  uint16_t* wo = a.ws_o + (part * kWaves + wave) * (int64_t)(4 * 16 * 64);
   const float inv_l = l_tot == 0.0f ? 0.0f : 1.0f / l_tot;
 #pragma unroll
-  for (int mt = 0; mt < 8; mt++)
+  for (int mt = 0; mt < 4; mt++)
 #pragma unroll
     for (int c = 0; c < 4; c += 2) {
       uint32_t w[4];
@@ -677,14 +701,14 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int c = tid >> 6;  // accumulator quad: registers 4c..4c+3 (half of a stored group of 8)
-  const int mt = blockIdx.x & 7;
-  const int wave = (blockIdx.x >> 3) & 3;
+  const int mt = blockIdx.x & 3;
+  const int wave = (blockIdx.x >> 2) & 7;  // wave of the split kernel whose registers this workgroup merges
   const int bh = blockIdx.x >> 5;
   const int hb = bh % a.n_hblk;
   const int seq = bh / a.n_hblk;
   const int b = seq / a.n_tokens;
   const int t = seq - b * a.n_tokens;
-  const int hg = wave >> 1, dh = wave & 1;
+  const int hg = wave >> 2, dh = wave & 3;
   const int n = lane & 31, g = lane >> 5;
   const int head = hb * 64 + hg * 32 + n;
   if (head >= a.n_heads) return;
@@ -693,7 +717,7 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   const int64_t part0 = (int64_t)(seq * a.n_hblk + hb) * a.n_splits;
   const float* ml0 = a.ws_ml + (part0 * 64 + hg * 32 + n) * 2;
   const uint16_t* wo0 =
-      a.ws_o + (part0 * 4 + wave) * (int64_t)(8 * 16 * 64) + ((mt * 2 + c / 2) * 64 + lane) * 8 + (c & 1) * 4;
+      a.ws_o + (part0 * kWaves + wave) * (int64_t)(4 * 16 * 64) + ((mt * 2 + c / 2) * 64 + lane) * 8 + (c & 1) * 4;
   // One online pass in chunks of 16 ranges: the statistics and the partial rows of a chunk are all
   // requested at once, so a sequence split into up to 16 ranges costs one memory round trip.
   constexpr int kChunk = 16;
@@ -729,7 +753,7 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   }
   const float inv = l == 0.0f ? 0.0f : 1.0f / l;
   float r[4] = {o.x * inv, o.y * inv, o.z * inv, o.w * inv};
-  const int dim0 = dh * 256 + 32 * mt + 8 * c + 4 * g;
+  const int dim0 = dh * 128 + 32 * mt + 8 * c + 4 * g;
   const int64_t ooff = (int64_t)b * a.out_batch_stride + (int64_t)t * a.out_token_stride +
                        (int64_t)head * a.out_head_stride + dim0;
   emit_output<ODT>(a, r, ooff, dim0);
