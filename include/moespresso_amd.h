@@ -178,6 +178,17 @@ int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, c
                            int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
                            float scale, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Partial rotary embedding of the last 64 channels of rows laid out [n_outer, seq_len, width]
+ * (interleaved pairs); the leading channels copy through.
+ * Replaces fused_partial_rope, runtime/deepseek_v4/attention_seam_kernel.py:247 (the composed
+ * _apply_partial_rope sequence at element-type rounding; kernel source :80-118).
+ * x/out: dtype f32|f16|bf16, 16-byte aligned; inv_freq: float32 [32]; positions: float32 [seq_len] or
+ * NULL (then row l of the sequence axis sits at position offset + l, offset + seq_len <= 2^24);
+ * inverse != 0 negates the sine. */
+int mspr_fused_partial_rope(const void* x, int dtype, int64_t n_outer, int64_t seq_len, int width,
+                            const float* inv_freq, const float* positions, int64_t offset, int inverse,
+                            void* out, void* stream);
+
 /* ------------------------------------------------------------------ Qwen/Ornith GQA attention, 8-bit KV */
 
 /* Affine 8-bit quantisation in groups of 64 over the last axis and its inverse: the cache write

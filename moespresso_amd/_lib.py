@@ -53,6 +53,8 @@ SIGNATURES = {
     "mspr_sparse_mla_decode": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int64, c_int,
                 c_int, c_int, c_int64, c_int, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mspr_fused_partial_rope": (
+        c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p]),
     "mspr_affine_q8_quantize": (
         c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "mspr_affine_q8_dequantize": (

@@ -67,10 +67,11 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
 }
 
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
-  _Float16 h = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
-  uint16_t b;
-  __builtin_memcpy(&b, &h, 2);
-  return b;
+  // v_cvt_f16_f32 (round to nearest even), written out so that the compiler cannot merge a preceding
+  // float32 multiply into v_fma_mixlo_f16 with a +0 addend: that form turns a product of -0 into +0
+  uint32_t r;
+  asm("v_cvt_f16_f32 %0, %1" : "=v"(r) : "v"(f));
+  return (uint16_t)r;
 }
 
 // Load element i of a row stored as f32 / f16 / bf16, widened to float32 (exact).

@@ -604,6 +604,25 @@ def partial_rope_lowp(x: np.ndarray, pos: int, inv_freq: np.ndarray, *, inverse:
     return out
 
 
+def fused_partial_rope(x: np.ndarray, inv_freq: np.ndarray, *, offset: int = 0, inverse: bool = False,
+                       positions=None, dtype: str = "float32") -> np.ndarray:
+    """Partial rope of ``[..., seq, width]`` rows, one position per sequence row.
+
+    attention_seam_kernel.py:80-118 (kernel body) and :247-288 (operand forms): row ``r`` of the
+    flattened rows sits at ``offset + r % seq`` (offset form) or ``positions[r % seq]`` (positions
+    form, float32). ``dtype`` names the element type whose rounding every product and sum takes
+    ("float32", "float16", "bfloat16"); ``x`` holds values of that type as float32.
+    """
+    rnd = {"float32": lambda v: np.asarray(v, dtype=F32), "float16": round_f16, "bfloat16": round_bf16}[dtype]
+    x = np.asarray(x, dtype=F32)
+    seq = x.shape[-2]
+    out = np.empty_like(x)
+    for l in range(seq):
+        pos = F32(offset + l) if positions is None else F32(np.asarray(positions, dtype=F32).reshape(-1)[l])
+        out[..., l, :] = partial_rope_lowp(x[..., l, :], pos, inv_freq, inverse=inverse, rnd=rnd)
+    return out
+
+
 # --------------------------------------------------------------------------
 # A4: indexed mixed attention (visit rules + sink softmax)
 # --------------------------------------------------------------------------

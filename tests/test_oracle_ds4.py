@@ -299,6 +299,56 @@ def test_lowp_rope_tracks_float64_rope():
 
 # ---------------------------------------------------------------- attention
 
+_YARN = {"factor": 16.0, "original_seq_len": 65536, "beta_fast": 32, "beta_slow": 1}
+
+
+def test_fused_partial_rope_float32_tracks_float64_rope_and_copies_the_head():
+    # pins: the float64 closed form of attention.py:117-156; leading channels and signed zeros untouched
+    rng = np.random.default_rng(5)
+    x = (2.0 * rng.standard_normal((2, 5, 7, 128))).astype(np.float32)
+    x[0, 0, 0, :4] = -0.0
+    inv = ds4.rope_inverse_frequencies(64, 160000.0, _YARN).astype(np.float32)
+    for offset, inverse in ((0, False), (3855, True)):
+        got = ds4.fused_partial_rope(x, inv, offset=offset, inverse=inverse)
+        want = ds4.apply_rope_tail(x.astype(np.float64), np.arange(offset, offset + 7), base=160000.0, yarn=_YARN,
+                                   inverse=inverse)
+        np.testing.assert_array_equal(got[..., :64].view(np.uint32), x[..., :64].view(np.uint32))
+        # float32 angles lose about |theta| * 2^-24: a few 1e-4 at position 3855 on values up to ~8
+        assert np.abs(got - want).max() < (2e-5 if offset == 0 else 4e-3)
+    # offset form == positions form on the same positions; inverse undoes forward
+    pos = np.arange(40, 47, dtype=np.float32)
+    a = ds4.fused_partial_rope(x, inv, offset=40)
+    b = ds4.fused_partial_rope(x, inv, positions=pos)
+    np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+    back = ds4.fused_partial_rope(a, inv, offset=40, inverse=True)
+    assert np.abs(back - x).max() < 2e-6 * 8
+
+
+def test_fused_partial_rope_16bit_rounds_every_operation():
+    # pin: the same rotation carried out in NumPy's native float16 arithmetic, which rounds each
+    # product and sum to float16 by construction
+    rng = np.random.default_rng(6)
+    x16 = (2.0 * rng.standard_normal((3, 4, 512))).astype(np.float16)
+    inv = ds4.rope_inverse_frequencies(64, 10000.0).astype(np.float32)
+    offset = 17
+    got = ds4.fused_partial_rope(x16.astype(np.float32), inv, offset=offset, dtype="float16")
+    want = x16.copy()
+    for l in range(4):
+        theta = (np.float32(offset + l) * inv).astype(np.float32)
+        c = np.cos(theta.astype(np.float64)).astype(np.float32).astype(np.float16)
+        s = np.sin(theta.astype(np.float64)).astype(np.float32).astype(np.float16)
+        x0, x1 = x16[:, l, 448::2], x16[:, l, 449::2]
+        want[:, l, 448::2] = x0 * c - x1 * s
+        want[:, l, 449::2] = x0 * s + x1 * c
+    np.testing.assert_array_equal(got.astype(np.float16).view(np.uint16), want.view(np.uint16))
+    # bfloat16: results are bfloat16 values and stay within one bfloat16 step of the float32 rotation
+    xb = ds4.round_bf16((2.0 * rng.standard_normal((2, 3, 128))).astype(np.float32))
+    gb = ds4.fused_partial_rope(xb, inv, offset=3, dtype="bfloat16")
+    np.testing.assert_array_equal(gb.view(np.uint32), ds4.round_bf16(gb).view(np.uint32))
+    g32 = ds4.fused_partial_rope(xb, inv, offset=3)
+    assert np.abs(gb - g32).max() <= 2.0 ** -7 * np.abs(g32).max()
+
+
 def test_sink_attention_known_answer_and_softmax_limit():
     # reference tests/test_deepseek_v4_attention.py:146-160
     scores = np.array([[0.25]])
