@@ -234,14 +234,14 @@ def topk_select(scores: torch.Tensor, topk: int) -> torch.Tensor:
     337-375``).
 
     Args:
-        scores: float32 ``[n_rows]`` or ``[batch, n_rows]``.
+        scores: float32 ``[..., n_rows]``; the selection runs over the last axis.
         topk: ``0 < topk <= n_rows``.
 
     Returns:
-        int32 ``[topk]`` or ``[batch, topk]``.
+        int32 ``[..., topk]``.
     """
-    if scores.ndim not in (1, 2):
-        raise ValueError("scores must be [n_rows] or [batch, n_rows]")
+    if scores.ndim < 1:
+        raise ValueError("scores must have a row axis")
     if scores.dtype != torch.float32:
         raise ValueError("scores must be float32")
     n_rows = int(scores.shape[-1])

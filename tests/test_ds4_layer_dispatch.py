@@ -1,0 +1,80 @@
+"""Eligibility order of the fused ratio-4 decode wrapper on CPU tensors (no kernel runs): every miss
+delegates to the wrapped block before any cache mutation (reference model.py:1551-1607; test
+tests/test_deepseek_v4_decode_attention_kernel.py:532-578)."""
+
+import torch
+
+from ds4_standins import Attention, Cache, OtherCache, steady_cache
+from moespresso_amd.runtime.deepseek_v4 import decode_attention_kernel as dak
+from moespresso_amd.runtime.deepseek_v4 import model as dsm
+
+
+def _marked(**kw):
+    cache = steady_cache("cpu", **kw)
+    object.__setattr__(cache, "_moespresso_dsv4_fp8_kv_cache", True)
+    return cache
+
+
+def test_every_contract_miss_delegates_before_touching_the_cache(monkeypatch):
+    monkeypatch.setattr(dak, "fused_decode_enabled", lambda: True)
+    attn = Attention("cpu")
+    wrapper = dsm._Ratio4DecodeFusedAttention(attn, cache_cls=Cache)
+    x = torch.zeros((1, 1, 256), dtype=torch.float16)
+    good = _marked(rows=96)
+    assert wrapper._decode_eligible(x, good)
+
+    misses = []
+    misses.append((torch.zeros((1, 4, 256), dtype=torch.float16), good))          # prefill shape
+    misses.append((torch.zeros((2, 1, 256), dtype=torch.float16), good))          # batch
+    misses.append((x.float(), good))                                              # element type
+    misses.append((x, steady_cache("cpu", rows=96)))                              # cache without the rounded append
+    misses.append((x, _marked(rows=96, cls=OtherCache)))                          # another cache class
+    misses.append((x, _marked(rows=96, offset=100)))                              # ring not yet full
+    odd_keep = _marked(rows=96)
+    odd_keep.local.keep = 4
+    misses.append((x, odd_keep))                                                  # ring keeps a prefix
+    f32_ring = _marked(rows=96)
+    f32_ring.local.keys = f32_ring.local.keys.float()
+    misses.append((x, f32_ring))                                                  # ring element type
+    short = _marked(rows=96)
+    short.local.max_size = 64
+    misses.append((x, short))                                                     # ring size != sliding window
+    for xi, cache in misses:
+        assert not wrapper._decode_eligible(xi, cache)
+        wrapper(xi, mask=None, cache=cache)
+    assert len(attn.stock_calls) == len(misses)
+    assert attn.compressor.calls == [] and wrapper.fused_decode_calls == 0
+
+    # geometry of the wrapped block
+    for name, value in (("compress_ratio", 128), ("head_dim", 256)):
+        other = Attention("cpu")
+        setattr(other, name, value)
+        assert not dsm._Ratio4DecodeFusedAttention(other, cache_cls=Cache)._decode_eligible(x, good)
+    other = Attention("cpu")
+    other.indexer.index_topk = 0
+    assert not dsm._Ratio4DecodeFusedAttention(other, cache_cls=Cache)._decode_eligible(x, good)
+    other = Attention("cpu")
+    other.rope.dims = 32
+    assert not dsm._Ratio4DecodeFusedAttention(other, cache_cls=Cache)._decode_eligible(x, good)
+
+    # debug dumps veto the fused path; the gate itself too
+    monkeypatch.setenv("MOESPRESSO_DSV4_INDEXER_DUMP_PREFIX", "/tmp/x")
+    assert not wrapper._decode_eligible(x, good)
+    monkeypatch.delenv("MOESPRESSO_DSV4_INDEXER_DUMP_PREFIX")
+    monkeypatch.setattr(dak, "fused_decode_enabled", lambda: False)
+    assert not wrapper._decode_eligible(x, good)
+
+
+def test_cache_wrappers_are_idempotent_and_keep_the_originals():
+    cache = steady_cache("cpu", rows=4)
+    original = cache.update_and_fetch
+    dsm._cache_with_fp8_kv_roundtrip(cache)
+    dsm._cache_with_fp8_kv_roundtrip(cache)
+    assert getattr(cache, dsm._CACHE_WRAPPER_ORIGINALS_ATTR)["update_and_fetch"] == original
+    dsm._cache_with_compressed_pool_aux_trim_clear(cache)
+    dsm._cache_with_compressed_pool_aux_trim_clear(cache)
+    assert set(getattr(cache, dsm._CACHE_WRAPPER_ORIGINALS_ATTR)) == {"update_and_fetch", "trim"}
+    # rows of another width pass through the wrapped update untouched (no kernel involved)
+    rows = torch.zeros((1, 1, 2, 128))
+    k, v = cache.update_and_fetch(rows, rows)
+    assert k is rows and v is rows and cache.update_calls == 1

@@ -1,0 +1,238 @@
+"""GPU tests of the DS4 layer glue: cache write path, pooled-row QAT cache, decode score contract and
+the fused ratio-4 decode attention wrapper, against the NumPy oracle of the two fused kernels.
+
+The cases follow the reference's wrapper tests (tests/test_deepseek_v4_decode_attention_kernel.py
+:184-212, :459-578); the composed layer they compare against needs third-party packages, so the oracle
+of the fused pair (pinned elsewhere) stands in for it, fed with the projections the wrapper itself saw.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from moespresso_amd.runtime.deepseek_v4 import decode_attention_kernel as dak
+from moespresso_amd.runtime.deepseek_v4 import indexer_score_kernel as isk
+from moespresso_amd.runtime.deepseek_v4 import model as dsm
+from oracle import ds4
+from ds4_standins import OFFSET, Attention, Cache, OtherCache, steady_cache
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy()
+
+
+def _run_fused(monkeypatch, *, rows=96, idx=37):
+    monkeypatch.setattr(dak, "_ENABLED", True)
+    attn = Attention(DEV)
+    wrapper = dsm._Ratio4DecodeFusedAttention(attn, cache_cls=Cache)
+    cache = dsm._cache_with_fp8_kv_roundtrip(steady_cache(DEV, rows=rows, idx=idx))
+    x = (torch.randn((1, 1, 256), generator=torch.Generator().manual_seed(5)) * 0.05).to(torch.float16).to(DEV)
+    seen = {}
+    real_prep, real_sdpa = dak.fused_decode_prep, dak.fused_decode_sdpa
+
+    def prep(*a, **k):
+        seen["prep_in"] = (a, k)
+        seen["prep_out"] = real_prep(*a, **k)
+        return seen["prep_out"]
+
+    def sdpa(*a, **k):
+        seen["sdpa_in"] = (tuple(t.clone() for t in a), k)  # the window is a view of the ring, appended to later
+        return real_sdpa(*a, **k)
+
+    monkeypatch.setattr(dak, "fused_decode_prep", prep)
+    monkeypatch.setattr(dak, "fused_decode_sdpa", sdpa)
+    window_before = cache.local.keys.clone()
+    out = wrapper(x, mask=None, cache=cache)
+    torch.cuda.synchronize()
+    return attn, wrapper, cache, x, out, seen, window_before
+
+
+def test_fused_decode_wrapper_matches_oracle_of_the_fused_pair(monkeypatch):
+    attn, wrapper, cache, x, out, seen, window_before = _run_fused(monkeypatch)
+    assert wrapper.fused_decode_calls == 1 and wrapper.fused_decode_composed_tail_calls == 0
+    assert attn.stock_calls == [] and attn.tail_calls == []
+    # both compressors advanced once, the indexer one on its own state
+    assert attn.compressor.calls == ["compressor_state"] and attn.indexer.compressor.calls == ["indexer_state"]
+
+    (q_idx, pooled_qat, weights, kv_row, inv, params), kw = seen["prep_in"]
+    assert kw == {"scale": 128 ** -0.5, "topk": 64}
+    assert params.cpu().tolist() == [OFFSET, 37]
+    sel, row, scores = seen["prep_out"]
+    # the pooled QAT rows are the kernel's QAT of the indexer pool, kept in the cache state
+    np.testing.assert_array_equal(_np(pooled_qat), ds4.indexer_qat(_np(cache.indexer_state["pooled"][0])))
+    assert cache.indexer_state["pooled_qat_rows"] == 96
+    # prepared row and selection against the oracle (selection on the device's own scores)
+    o_sel, o_row, o_scores = ds4.fused_decode_prep(_np(q_idx), _np(pooled_qat), _np(weights), _np(kv_row), _np(inv),
+                                                   params.cpu().numpy(), scale=128 ** -0.5, topk=64)
+    np.testing.assert_array_equal(_np(row).astype(np.float16).view(np.uint16), o_row.astype(np.float16).view(np.uint16))
+    np.testing.assert_allclose(_np(scores), o_scores, rtol=2e-5, atol=2e-5)
+    np.testing.assert_array_equal(sel.cpu().numpy(), ds4.radix_select_topk(_np(scores), 64))
+
+    (q, window, row_in, pooled, sel_in, sinks, inv2, params2), kw2 = seen["sdpa_in"]
+    np.testing.assert_array_equal(_np(window), _np(window_before[0, 0]))  # the ring as it stood before the append
+    want = ds4.fused_decode_sdpa(_np(q), _np(window), _np(row_in), _np(pooled), sel_in.cpu().numpy(), _np(sinks),
+                                 _np(inv2), params2.cpu().numpy(), scale=512 ** -0.5).astype(np.float32)
+    got = _np(attn.heads_seen).reshape(8, 512)
+    assert np.abs(got - want).max() < 2e-3
+    np.testing.assert_array_equal(_np(out), _np(attn.wo_b(attn.heads_seen)))
+
+    # direct append: ring slot 37 holds the prepared row in keys and values, counters moved by one
+    assert cache.local.offset == OFFSET + 1 and cache.local._idx == 38
+    np.testing.assert_array_equal(_np(cache.local.keys[0, 0, 37]), _np(row))
+    np.testing.assert_array_equal(_np(cache.local.values[0, 0, 37]), _np(row))
+    untouched = [i for i in range(128) if i != 37]
+    np.testing.assert_array_equal(_np(cache.local.keys[0, 0, untouched]), _np(window_before[0, 0, untouched]))
+    assert cache.update_calls == 0  # the rounded append bypasses update_and_fetch
+
+
+def test_fused_decode_wrapper_wraps_the_ring_write_slot(monkeypatch):
+    attn, wrapper, cache, x, out, seen, _ = _run_fused(monkeypatch, idx=128)
+    (_, _, _, _, _, params), _ = seen["prep_in"]
+    assert params.cpu().tolist() == [OFFSET, 0]
+    assert cache.local._idx == 1
+    np.testing.assert_array_equal(_np(cache.local.keys[0, 0, 0]), _np(seen["prep_out"][1]))
+
+
+def test_fused_decode_wrapper_hands_short_pools_to_the_composed_tail(monkeypatch):
+    attn, wrapper, cache, x, out, seen, window_before = _run_fused(monkeypatch, rows=32)
+    assert wrapper.fused_decode_calls == 0 and wrapper.fused_decode_composed_tail_calls == 1
+    assert "prep_in" not in seen
+    (kw,) = attn.tail_calls
+    assert kw["run_indexer"] is True and kw["topk"] is None and kw["offset"] == OFFSET
+    assert tuple(kw["q"].shape) == (1, 1, 8, 512) and tuple(kw["kv"].shape) == (1, 1, 1, 512)
+    # nothing was appended by the wrapper itself
+    np.testing.assert_array_equal(_np(cache.local.keys), _np(window_before))
+    assert cache.local.offset == OFFSET
+
+
+def test_fused_decode_wrapper_without_a_tail_fails_loudly(monkeypatch):
+    monkeypatch.setattr(dak, "_ENABLED", True)
+    attn = Attention(DEV)
+    attn.composed_decode_tail = None
+    wrapper = dsm._Ratio4DecodeFusedAttention(attn, cache_cls=Cache)
+    cache = dsm._cache_with_fp8_kv_roundtrip(steady_cache(DEV, rows=32))
+    x = torch.zeros((1, 1, 256), dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="composed_decode_tail"):
+        wrapper(x, mask=None, cache=cache)
+
+
+def test_fused_decode_wrapper_delegates_outside_contract(monkeypatch):
+    attn = Attention(DEV)
+    wrapper = dsm._Ratio4DecodeFusedAttention(attn, cache_cls=Cache)
+    x = torch.zeros((1, 1, 256), dtype=torch.float16, device=DEV)
+    cache = steady_cache(DEV, rows=96)
+    monkeypatch.setattr(dak, "_ENABLED", False)                      # gate off
+    wrapper(x, mask=None, cache=dsm._cache_with_fp8_kv_roundtrip(steady_cache(DEV, rows=96)))
+    monkeypatch.setattr(dak, "_ENABLED", True)
+    wrapper(x, mask=None, cache=cache)                               # no rounded-append contract on the cache
+    marked = dsm._cache_with_fp8_kv_roundtrip(steady_cache(DEV, rows=96))
+    wrapper(torch.zeros((1, 4, 256), dtype=torch.float16, device=DEV), mask=None, cache=marked)  # prefill shape
+    wrapper(x.float(), mask=None, cache=marked)                      # element type
+    wrapper(x, mask=None, cache=dsm._cache_with_fp8_kv_roundtrip(steady_cache(DEV, rows=96, cls=OtherCache)))
+    cold = dsm._cache_with_fp8_kv_roundtrip(steady_cache(DEV, rows=96, offset=100))
+    wrapper(x, mask=None, cache=cold)                                # ring not yet full
+    wrapper(x, mask=None, cache=None)
+    assert len(attn.stock_calls) == 7
+    assert wrapper.fused_decode_calls == 0 and attn.compressor.calls == []
+
+
+def test_patch_installs_fused_decode_wrapper_by_gate(monkeypatch):
+    from types import SimpleNamespace
+    layers = [SimpleNamespace(attn=Attention(DEV)), SimpleNamespace(attn=SimpleNamespace(compress_ratio=128)),
+              SimpleNamespace()]
+    model = SimpleNamespace(model=SimpleNamespace(layers=layers))
+    monkeypatch.setattr(dak, "_ENABLED", False)
+    assert dsm._patch_deepseek_v4_ratio4_decode_fused_attention(model, cache_cls=Cache) == 0
+    monkeypatch.setattr(dak, "_ENABLED", True)
+    assert dsm._patch_deepseek_v4_ratio4_decode_fused_attention(model, cache_cls=Cache) == 1
+    assert isinstance(layers[0].attn, dsm._Ratio4DecodeFusedAttention)
+    assert dsm._patch_deepseek_v4_ratio4_decode_fused_attention(model, cache_cls=Cache) == 0  # idempotent
+    assert layers[0].attn.n_heads == 8  # attributes of the wrapped block stay reachable
+
+
+def test_fp8_cache_write_path_rounds_rows_once(monkeypatch):
+    cache = steady_cache(DEV, rows=8)
+    wrapped = dsm._cache_with_fp8_kv_roundtrip(cache)
+    assert wrapped is cache and cache._moespresso_dsv4_fp8_kv_cache
+    assert dsm._cache_with_fp8_kv_roundtrip(cache) is cache  # idempotent: still one layer of rounding
+    rng = np.random.default_rng(3)
+    rows = torch.from_numpy(rng.standard_normal((1, 1, 5, 512), dtype=np.float32)).to(DEV)
+    k, v = cache.update_and_fetch(rows, rows)
+    assert cache.update_calls == 1 and k is v
+    np.testing.assert_array_equal(_np(k), ds4.fp8_kv_roundtrip(_np(rows)))
+    k2, v2 = cache.update_and_fetch(rows, rows.clone())
+    np.testing.assert_array_equal(_np(v2), _np(k2))
+    # 16-bit rows: float32 arithmetic, cast back
+    half = rows.to(torch.float16)
+    kh, _ = cache.update_and_fetch(half, half)
+    assert kh.dtype == torch.float16
+    np.testing.assert_array_equal(_np(kh), ds4.fp8_kv_roundtrip(_np(half)).astype(np.float16).astype(np.float32))
+    # rows of another width and empty tensors pass through
+    odd = torch.zeros((1, 1, 2, 128), device=DEV)
+    assert dsm._deepseek_v4_fp8_kv_roundtrip(odd) is odd
+    with pytest.raises(dsm.DeepseekV4RuntimeLoadError):
+        dsm._deepseek_v4_fp8_kv_roundtrip(torch.zeros((2, 96), device=DEV), head_dim=96, rot_dim=64)
+
+
+def test_trim_clears_the_derived_pool_caches():
+    cache = dsm._cache_with_compressed_pool_aux_trim_clear(steady_cache(DEV, rows=8))
+    cache.indexer_state.update(pooled_qat=1, pooled_qat_rows=8)
+    cache.compressor_state.update(pooled_fp8=1, pooled_fp8_rows=8)
+    assert cache.trim(3) == 3 and cache.trim_calls == 1
+    assert "pooled_qat" not in cache.indexer_state and "pooled_qat_rows" not in cache.indexer_state
+    assert "pooled_fp8" not in cache.compressor_state and "pooled" in cache.compressor_state
+
+
+def test_pooled_qat_update_is_incremental_and_bit_equal_to_a_full_pass():
+    rng = np.random.default_rng(8)
+    pool = torch.from_numpy(rng.standard_normal((1, 40, 128), dtype=np.float32)).to(torch.float16).to(DEV)
+    state = {}
+    a, cached, new = dsm.pooled_qat_update(state, pool[:, :24])
+    assert (cached, new) == (0, 24) and state["pooled_qat_rows"] == 24
+    b, cached, new = dsm.pooled_qat_update(state, pool[:, :24])
+    assert (cached, new) == (24, 0) and b is a
+    c, cached, new = dsm.pooled_qat_update(state, pool)
+    assert (cached, new) == (24, 16) and state["pooled_qat_rows"] == 40
+    np.testing.assert_array_equal(_np(c), _np(dsm._dsv4_indexer_qat(pool)))
+    np.testing.assert_array_equal(_np(c), ds4.indexer_qat(_np(pool)))
+    # a cache longer than the pool (after a trim) is not trusted
+    d, cached, new = dsm.pooled_qat_update({"pooled_qat": c, "pooled_qat_rows": 40}, pool[:, :10])
+    assert (cached, new) == (0, 10) and tuple(d.shape) == (1, 10, 128)
+    # without a state dict nothing is kept
+    e, cached, new = dsm.pooled_qat_update(None, pool[:, :3])
+    assert (cached, new) == (0, 3)
+
+
+def test_decode_score_contract_selects_on_the_fused_score_row(monkeypatch):
+    monkeypatch.setattr(isk, "_ENABLED", True)
+    attn = Attention(DEV, index_heads=64, topk=16)
+    contract = dsm._IndexerDS4ScoreContract(attn.indexer, 4, layer_index=0)
+    cache = steady_cache(DEV, rows=200)
+    x = (torch.randn((1, 1, 256), generator=torch.Generator().manual_seed(2)) * 0.05).to(torch.float16).to(DEV)
+    q_res = attn.q_norm(attn.wq_a(x))
+    topk = contract(x, q_res, attn.compress_rope, attn.rope, cache, OFFSET)
+    assert tuple(topk.shape) == (1, 1, 16) and topk.dtype == torch.int32
+    # the same row through the kernels by hand
+    q = attn.indexer.wq_b(q_res).reshape(1, 1, 64, 128).transpose(1, 2)
+    from moespresso_amd.runtime.deepseek_v4 import attention_seam_kernel as seam
+    q = seam.fused_partial_rope(q, attn.rope.inv_freq, offset=OFFSET)
+    w = attn.indexer.weights_proj(x).float() * 64 ** -0.5
+    scores = isk.fused_qat_indexer_scores(q, cache.indexer_state["pooled_qat"], w, 128 ** -0.5)
+    np.testing.assert_array_equal(topk.cpu().numpy().reshape(-1), ds4.radix_select_topk(_np(scores), 16))
+    o_scores = ds4.fused_qat_indexer_scores(_np(q), _np(cache.indexer_state["pooled_qat"]), _np(w), 128 ** -0.5)
+    np.testing.assert_allclose(_np(scores), o_scores.reshape(-1), rtol=2e-5, atol=2e-5)
+    c = "_moespresso_dsv4_indexer_score_contract_"
+    assert getattr(contract, c + "calls") == 1 and getattr(contract, c + "fused_score_calls") == 1
+    assert getattr(contract, c + "new_qat_pooled_rows") == 200 and getattr(contract, c + "topk_rows") == 16
+    # second token: the pool rows are reused
+    contract(x, q_res, attn.compress_rope, attn.rope, cache, OFFSET + 1)
+    assert getattr(contract, c + "cached_pooled_rows") == 200 and getattr(contract, c + "new_qat_pooled_rows") == 200
+    # prefill shapes go to the wrapped indexer, and so does a decode token while the score gate is off
+    contract(torch.zeros((1, 4, 256), dtype=torch.float16, device=DEV), q_res, None, None, cache, 0)
+    assert attn.indexer.stock_calls == 1
+    monkeypatch.setattr(isk, "_ENABLED", False)
+    assert contract(x, q_res, attn.compress_rope, attn.rope, cache, OFFSET + 2) is None
+    assert attn.indexer.stock_calls == 2
