@@ -13,7 +13,8 @@ Mirror of the attention-path pieces of the reference module
 - ``_IndexerDS4ScoreContract`` (:833): the decode-shaped branch (QAT'd query and pool, fused score
   row, deterministic top-k);
 - ``_Ratio4DecodeFusedAttention`` (:1519): eligibility (:1551-1607), the two fused launches and the
-  direct ring append (:1756-1789).
+  direct ring append (:1756-1789);
+- ``_Ratio4PrefillFastAttention`` (:1305): the prefill chunk through the live-layout kernels.
 
 The wrapped blocks are the model's own modules (torch here). Everything outside the fused contract
 goes to the wrapped block: an ineligible call is the block's own ``__call__``; a call that fails a
@@ -373,25 +374,135 @@ class _Ratio4DecodeFusedAttention:
         return attn.wo_b(out)
 
 
+def _attention_layers(model):
+    return getattr(getattr(model, "model", model), "layers", None) or ()
+
+
 def _patch_deepseek_v4_ratio4_decode_fused_attention(model, *, cache_cls) -> int:
     """Wrap the ratio-4 attention blocks of ``model``; returns how many were wrapped (reference :1792).
 
     Nothing is installed while the fused decode gate is off. Layers are found under ``model.layers``
-    (or ``model.model.layers``); a layer takes part when its ``attn`` block has ``compress_ratio == 4``
-    and an indexer.
+    (or ``model.model.layers``); a layer takes part when its ``self_attn`` block has
+    ``compress_ratio == 4`` and an indexer. The count is also left on the model.
     """
     if not decode_attention_kernel.fused_decode_enabled():
-        return 0
-    layers = getattr(getattr(model, "model", model), "layers", None)
-    if layers is None:
+        object.__setattr__(model, "_moespresso_dsv4_fused_decode_attention_layers", 0)
         return 0
     patched = 0
-    for layer in layers:
-        attn = getattr(layer, "attn", None)
+    for layer in _attention_layers(model):
+        attn = getattr(layer, "self_attn", None)
         if attn is None or getattr(attn, "_moespresso_dsv4_fused_decode_attention", False):
             continue
         if int(getattr(attn, "compress_ratio", 0) or 0) != 4 or not hasattr(attn, "indexer"):
             continue
-        layer.attn = _Ratio4DecodeFusedAttention(attn, cache_cls=cache_cls)
+        object.__setattr__(layer, "self_attn", _Ratio4DecodeFusedAttention(attn, cache_cls=cache_cls))
         patched += 1
+    object.__setattr__(model, "_moespresso_dsv4_fused_decode_attention_layers", patched)
+    return patched
+
+
+# ---------------------------------------------------------------- ratio-4 prefill fast path
+
+def _dsv4_prefill_pooled_qat(x: torch.Tensor) -> torch.Tensor:
+    """QAT of pooled indexer rows on the prefill path (reference :752); same kernel as the decode side."""
+    return indexer_score_kernel.indexer_qat_rows(x)
+
+
+class _Ratio4PrefillFastAttention:
+    """DS4 ratio-4 prefill through the live-layout kernels (reference :1305).
+
+    Projections, norms, rope and cache update run through the wrapped block's own modules and the rope
+    seam; the indexer queries take the live QAT, the pool rows the pooled QAT cache, scores come from the
+    tiled score kernel, the selection is the deterministic top-k sorted ascending, and attention is the
+    indexed mixed prefill consumer on BHLD operands. Single-token calls, other ratios, other cache
+    classes and blocks without an indexer go to the wrapped block.
+    """
+
+    def __init__(self, original, *, cache_cls):
+        self._original = original
+        self._cache_cls = cache_cls
+        self._moespresso_dsv4_ratio4_prefill_fast_path = True
+        self._moespresso_dsv4_ratio4_prefill_fast_calls = 0
+        self._moespresso_dsv4_ratio4_prefill_fast_tokens = 0
+
+    def __getattr__(self, name: str):
+        return getattr(self._original, name)
+
+    def _attend(self, q, kv, pooled, topk, offset, out_dtype):
+        from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+        attn = self._original
+        if q.dtype == torch.float16:
+            consumer, q_in = iak.indexed_mixed_attention_prefill_live_f16, q
+        else:
+            consumer, q_in = iak.indexed_mixed_attention_prefill_live_f32, q.to(torch.float32)
+        heads = consumer(q_in, kv.to(torch.float16), pooled.to(torch.float16), topk, attn.attn_sink.to(torch.float32),
+                         pos0=offset, window=int(attn.args.sliding_window), ratio=int(attn.compress_ratio))
+        out = _seam.fused_partial_rope(heads, attn.rope.inv_freq, offset=offset, inverse=True)
+        batch, _, tokens, _ = out.shape
+        out = out.transpose(1, 2).reshape(batch, tokens, attn.n_heads * attn.head_dim)
+        # the consumer and the inverse rope run in float32; the projections take the block's element type
+        return attn.wo_b(attn._grouped_output_projection(out.to(out_dtype)))
+
+    def __call__(self, x, mask=None, cache=None):
+        from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+        attn = self._original
+        batch, tokens, _ = x.shape
+        if (int(tokens) <= 1 or int(batch) != 1 or int(getattr(attn, "compress_ratio", 0) or 0) != 4
+                or not isinstance(cache, self._cache_cls) or not hasattr(attn, "indexer")):
+            return attn(x, mask=mask, cache=cache)
+
+        offset = int(cache.offset)
+        q_residual = attn.q_norm(attn.wq_a(x))
+        q = attn.wq_b(q_residual).reshape(batch, tokens, attn.n_heads, attn.head_dim)
+        q = torch.nn.functional.rms_norm(q, (int(attn.head_dim),), weight=None, eps=float(attn.args.rms_norm_eps))
+        q = q.transpose(1, 2)
+        kv = attn.kv_norm(attn.wkv(x)).reshape(batch, tokens, 1, attn.head_dim).transpose(1, 2)
+        q = _seam.fused_partial_rope(q, attn.rope.inv_freq, offset=offset)
+        kv = _seam.fused_partial_rope(kv, attn.rope.inv_freq, offset=offset)
+        kv, _ = cache.update_and_fetch(kv, kv)
+
+        pooled = attn.compressor(x, attn.compress_rope, cache, offset)
+        n_pool = int(pooled.shape[1])
+        if n_pool <= 0:
+            topk = torch.zeros((batch, tokens, 0), dtype=torch.int32, device=x.device)
+            return self._attend(q, kv, pooled, topk, offset, x.dtype)
+
+        indexer = attn.indexer
+        if n_pool <= int(indexer.index_topk):
+            row_ids = torch.arange(n_pool, dtype=torch.int32, device=x.device)
+            topk = row_ids[None, None, :].expand(batch, tokens, n_pool).contiguous()
+        else:
+            index_pooled = indexer.compressor(x, attn.compress_rope, cache, offset, state_key="indexer_state")
+            q_idx = indexer.wq_b(q_residual).reshape(batch, tokens, indexer.n_heads, indexer.head_dim).transpose(1, 2)
+            q_idx = _seam.fused_partial_rope(q_idx, attn.rope.inv_freq, offset=offset)
+            q_idx = iak.indexer_q_qat_live(q_idx.to(torch.float32))
+            index_pooled_qat, _, _ = pooled_qat_update(getattr(cache, "indexer_state", None), index_pooled)
+            weights = indexer.weights_proj(x).to(torch.float32) * (int(indexer.n_heads) ** -0.5) * float(indexer.scale)
+            q_scores, comp_scores = iak.indexer_score_operands(q_idx, index_pooled_qat)
+            scores = iak.indexer_scores_tiled_live(q_scores, weights, comp_scores, pos0=offset,
+                                                   ratio=int(attn.compress_ratio))
+            topk_rows = min(int(indexer.index_topk), int(index_pooled_qat.shape[1]))
+            topk = indexer_score_kernel.topk_select(scores, topk_rows)
+            topk = torch.sort(topk, dim=-1).values.to(torch.int32)
+
+        out = self._attend(q, kv, pooled, topk, offset, x.dtype)
+        self._moespresso_dsv4_ratio4_prefill_fast_calls += 1
+        self._moespresso_dsv4_ratio4_prefill_fast_tokens += int(tokens)
+        return out
+
+
+def _patch_deepseek_v4_ratio4_prefill_fast_path(model, *, cache_cls) -> int:
+    """Install the ratio-4 prefill fast path on the layers of ``model`` (reference :1482)."""
+    patched = 0
+    for layer in _attention_layers(model):
+        attn = getattr(layer, "self_attn", None)
+        if attn is None or getattr(attn, "_moespresso_dsv4_ratio4_prefill_fast_path", False):
+            continue
+        if int(getattr(attn, "compress_ratio", 0) or 0) != 4 or not hasattr(attn, "indexer"):
+            continue
+        object.__setattr__(layer, "self_attn", _Ratio4PrefillFastAttention(attn, cache_cls=cache_cls))
+        patched += 1
+    object.__setattr__(model, "_moespresso_dsv4_ratio4_prefill_fast_path_layers", patched)
     return patched

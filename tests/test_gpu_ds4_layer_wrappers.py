@@ -141,16 +141,17 @@ def test_fused_decode_wrapper_delegates_outside_contract(monkeypatch):
 
 def test_patch_installs_fused_decode_wrapper_by_gate(monkeypatch):
     from types import SimpleNamespace
-    layers = [SimpleNamespace(attn=Attention(DEV)), SimpleNamespace(attn=SimpleNamespace(compress_ratio=128)),
+    layers = [SimpleNamespace(self_attn=Attention(DEV)), SimpleNamespace(self_attn=SimpleNamespace(compress_ratio=128)),
               SimpleNamespace()]
     model = SimpleNamespace(model=SimpleNamespace(layers=layers))
     monkeypatch.setattr(dak, "_ENABLED", False)
     assert dsm._patch_deepseek_v4_ratio4_decode_fused_attention(model, cache_cls=Cache) == 0
     monkeypatch.setattr(dak, "_ENABLED", True)
     assert dsm._patch_deepseek_v4_ratio4_decode_fused_attention(model, cache_cls=Cache) == 1
-    assert isinstance(layers[0].attn, dsm._Ratio4DecodeFusedAttention)
+    assert isinstance(layers[0].self_attn, dsm._Ratio4DecodeFusedAttention)
+    assert model._moespresso_dsv4_fused_decode_attention_layers == 1
     assert dsm._patch_deepseek_v4_ratio4_decode_fused_attention(model, cache_cls=Cache) == 0  # idempotent
-    assert layers[0].attn.n_heads == 8  # attributes of the wrapped block stay reachable
+    assert layers[0].self_attn.n_heads == 8  # attributes of the wrapped block stay reachable
 
 
 def test_fp8_cache_write_path_rounds_rows_once(monkeypatch):
@@ -236,3 +237,70 @@ def test_decode_score_contract_selects_on_the_fused_score_row(monkeypatch):
     monkeypatch.setattr(isk, "_ENABLED", False)
     assert contract(x, q_res, attn.compress_rope, attn.rope, cache, OFFSET + 2) is None
     assert attn.indexer.stock_calls == 2
+
+
+def _prefill_setup(tokens, rows, *, topk, q_dtype=torch.float16):
+    attn = Attention(DEV, topk=topk, index_heads=64)
+    wrapper = dsm._Ratio4PrefillFastAttention(attn, cache_cls=Cache)
+    cache = steady_cache(DEV, rows=rows, offset=0)
+    x = (torch.randn((1, tokens, 256), generator=torch.Generator().manual_seed(9)) * 0.05).to(torch.float16).to(DEV)
+    return attn, wrapper, cache, x
+
+
+@pytest.mark.parametrize("rows,topk", [(40, 64), (40, 16)])
+def test_prefill_fast_path_matches_oracle_of_the_consumer(rows, topk):
+    # 160 tokens from position 0: pool rows (q+1)//4 become visible as the chunk proceeds
+    from moespresso_amd.runtime.deepseek_v4 import attention_seam_kernel as seam
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+    tokens = 160
+    attn, wrapper, cache, x = _prefill_setup(tokens, rows, topk=topk)
+    out = wrapper(x, mask=None, cache=cache)
+    torch.cuda.synchronize()
+    assert wrapper._moespresso_dsv4_ratio4_prefill_fast_calls == 1
+    assert wrapper._moespresso_dsv4_ratio4_prefill_fast_tokens == tokens
+    assert cache.update_calls == 1 and attn.stock_calls == []
+
+    # the same chunk by hand up to the consumer, then the oracle of the consumer
+    q_res = attn.q_norm(attn.wq_a(x))
+    q = attn.wq_b(q_res).reshape(1, tokens, 8, 512)
+    q = torch.nn.functional.rms_norm(q, (512,), eps=1e-6).transpose(1, 2)
+    kv = attn.kv_norm(attn.wkv(x)).reshape(1, tokens, 1, 512).transpose(1, 2)
+    q = seam.fused_partial_rope(q, attn.rope.inv_freq, offset=0)
+    kv = seam.fused_partial_rope(kv, attn.rope.inv_freq, offset=0)
+    np.testing.assert_array_equal(_np(cache.last_update[0]), _np(kv))
+    pooled = cache.compressor_state["pooled"]
+    if rows <= topk:
+        ids = np.broadcast_to(np.arange(rows, dtype=np.int32), (tokens, rows))
+        assert attn.indexer.compressor.calls == []
+    else:
+        q_idx = attn.indexer.wq_b(q_res).reshape(1, tokens, 64, 128).transpose(1, 2)
+        q_idx = iak.indexer_q_qat_live(seam.fused_partial_rope(q_idx, attn.rope.inv_freq, offset=0).float())
+        w = attn.indexer.weights_proj(x).float() * 64 ** -0.5 * 128 ** -0.5
+        scores = iak.indexer_scores_tiled_live(q_idx, w, cache.indexer_state["pooled_qat"], pos0=0, ratio=4)
+        ids = np.stack([np.sort(ds4.radix_select_topk(_np(scores)[0, t], topk)) for t in range(tokens)]).astype(np.int32)
+        assert cache.indexer_state["pooled_qat_rows"] == rows
+    want = ds4.indexed_mixed_attention_prefill(_np(q)[0].transpose(1, 0, 2), _np(kv)[0, 0], _np(pooled)[0], ids,
+                                               _np(attn.attn_sink), pos0=0, window=128, ratio=4)       # [T, H, 512]
+    want_rot = ds4.fused_partial_rope(want.transpose(1, 0, 2).astype(np.float32), _np(attn.rope.inv_freq), offset=0,
+                                      inverse=True)                                                     # [H, T, 512]
+    heads = _np(attn.heads_seen).reshape(tokens, 8, 512).transpose(1, 0, 2)
+    assert attn.heads_seen.dtype == torch.float16
+    assert np.abs(heads - want_rot).max() < 2e-3
+    np.testing.assert_array_equal(_np(out), _np(attn.wo_b(attn.heads_seen)))
+
+
+def test_prefill_fast_path_delegates_outside_its_shapes():
+    attn, wrapper, cache, x = _prefill_setup(8, 40, topk=16)
+    wrapper(x[:, :1], mask=None, cache=cache)                                   # one token
+    wrapper(torch.cat([x, x]), mask=None, cache=cache)                          # batch 2
+    wrapper(x, mask=None, cache=steady_cache(DEV, rows=40, cls=OtherCache))     # another cache class
+    wrapper(x, mask=None, cache=None)
+    attn.compress_ratio = 128
+    wrapper(x, mask=None, cache=cache)
+    assert len(attn.stock_calls) == 5 and wrapper._moespresso_dsv4_ratio4_prefill_fast_calls == 0
+    assert cache.update_calls == 0
+    from types import SimpleNamespace
+    model = SimpleNamespace(layers=[SimpleNamespace(self_attn=Attention(DEV)), SimpleNamespace(self_attn=None)])
+    assert dsm._patch_deepseek_v4_ratio4_prefill_fast_path(model, cache_cls=Cache) == 1
+    assert dsm._patch_deepseek_v4_ratio4_prefill_fast_path(model, cache_cls=Cache) == 0
+    assert model._moespresso_dsv4_ratio4_prefill_fast_path_layers == 0
