@@ -36,7 +36,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel at batch 16 (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
 # the same counters' reading for a 1 GiB elementwise kernel; profiles/bench_sparse_decode_layer_hbm_counters.txt)
-SPLIT_TRAFFIC_BYTES_B16 = 75_350_000
+SPLIT_TRAFFIC_BYTES_B16 = 58_490_000
 
 # workload constants (BASELINE configs 4 and 5)
 N_IDX_HEADS, IDX_DIM, N_KEYS, TOPK = 64, 128, 32768, 2048
