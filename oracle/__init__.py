@@ -35,4 +35,9 @@ would fail; "unpinned" = only self-consistency is available):
                                      tests this kernel to 1e-5 only)
   indexer_scores_tiled_live          pinned  (term-by-term float64 sum on half-rounded operands,
                                      visibility against the closed form)
+  fused_partial_rope                 pinned  (float64 rope closed form, NumPy's native float16
+                                     arithmetic for the per-operation rounding, offset form ==
+                                     positions form, inverse undoes forward); parity unpinned in the
+                                     last bit of cos/sin: correctly rounded float32 here, Metal's
+                                     precise::cos/sin bits unknown
 """
