@@ -185,6 +185,49 @@ def bench_q8_decode(dev, gen, reps=40):
     return out
 
 
+def bench_ds4_prefill(dev, gen, reps=5):
+    """DS4 prefill-side operators at the reference's anchor chunk: 3844 tokens from position 0, 64 heads,
+    961 pool rows, top-512, window 128 (wall time per call from torch events on the current stream)."""
+    from moespresso_amd.runtime.deepseek_v4 import attention_seam_kernel as seam
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+    T, H, P = 3844, 64, 961
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ts = []
+        for _ in range(reps):
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        return round(float(np.median(ts)), 4)
+
+    q = torch.randn((1, H, T, 512), device=dev, generator=gen).to(torch.float16)
+    raw = torch.randn((1, 1, T, 512), device=dev, generator=gen).to(torch.float16)
+    comp = torch.randn((1, P, 512), device=dev, generator=gen).to(torch.float16)
+    ids = torch.stack([torch.sort(torch.randperm(P, device=dev, generator=gen)[:512]).values for _ in range(T)])
+    ids = ids[None].to(torch.int32).contiguous()
+    sinks = torch.randn((H,), device=dev, generator=gen)
+    qi = torch.randn((1, H, T, 128), device=dev, generator=gen).to(torch.float16)
+    ci = torch.randn((1, P, 128), device=dev, generator=gen).to(torch.float16)
+    w = torch.rand((1, T, H), device=dev, generator=gen)
+    inv = torch.rand((32,), device=dev, generator=gen)
+    out = {
+        "indexed_attention_ms": timed(lambda: iak.indexed_mixed_attention_prefill_live_f16(
+            q, raw, comp, ids, sinks, pos0=0, window=128, ratio=4)),
+        "tiled_scores_ms": timed(lambda: iak.indexer_scores_tiled_live(qi, w, ci, pos0=0, ratio=4)),
+        "live_qat_ms": timed(lambda: iak.indexer_q_qat_live(qi.float())),
+        "partial_rope_query_ms": timed(lambda: seam.fused_partial_rope(q, inv, offset=0)),
+        "workload": "3844-token chunk, 64 heads x 512, 961 pool rows, top-512, window 128 (float16 operands)",
+    }
+    out["partial_rope_GBps"] = round(2 * q.numel() * 2 / (out["partial_rope_query_ms"] * 1e-3) / 1e9, 1)
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -304,6 +347,7 @@ def main() -> int:
         "kernel_us_by_batch": by_batch,
         "prefill": None if args.headline_only else bench_prefill(dev, gen),
         "q8_decode": None if args.headline_only else bench_q8_decode(dev, gen),
+        "ds4_prefill": None if args.headline_only else bench_ds4_prefill(dev, gen),
         "cpu_config1": None if args.no_cpu_baseline else cpu_config1(),
         "indexer_fp8_GBps": round(IDX_BYTES_PER_SEQ * B / (kernel_us["indexer_fp8"] * 1e-6) / 1e9, 1),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
