@@ -78,3 +78,21 @@ def test_cache_wrappers_are_idempotent_and_keep_the_originals():
     rows = torch.zeros((1, 1, 2, 128))
     k, v = cache.update_and_fetch(rows, rows)
     assert k is rows and v is rows and cache.update_calls == 1
+
+
+def test_replay_case_selection_and_rope_frequencies():
+    import numpy as np
+
+    from moespresso_amd.runtime.deepseek_v4 import ratio4_attention_replay as replay
+    from oracle import ds4
+
+    cases = replay.default_replay_cases()
+    assert [c.pooled_rows for c in cases] == [0, 961, 7618, 961, 512] and not cases[0].cache
+    assert replay.selected_replay_cases(include_splits=False) == cases[:3]
+    assert replay.selected_replay_cases(include_splits=True) == cases
+    picked = replay.selected_replay_cases(include_splits=False, pooled_rows=[100, 200], index_topk=64)
+    assert [c.name for c in picked] == ["ratio4_rows100_topk64", "ratio4_rows200_topk64"]
+    yarn = {"factor": 16.0, "original_seq_len": 65536, "beta_fast": 32, "beta_slow": 1}
+    for base, y in ((10000.0, None), (160000.0, yarn)):
+        np.testing.assert_array_equal(replay.rope_inverse_frequencies(64, base, y).numpy(),
+                                      ds4.rope_inverse_frequencies(64, base, y).astype(np.float32))

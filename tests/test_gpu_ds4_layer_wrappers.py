@@ -304,3 +304,37 @@ def test_prefill_fast_path_delegates_outside_its_shapes():
     assert dsm._patch_deepseek_v4_ratio4_prefill_fast_path(model, cache_cls=Cache) == 1
     assert dsm._patch_deepseek_v4_ratio4_prefill_fast_path(model, cache_cls=Cache) == 0
     assert model._moespresso_dsv4_ratio4_prefill_fast_path_layers == 0
+
+
+def test_one_layer_replay_reports_cases_and_stages():
+    from moespresso_amd.runtime.deepseek_v4 import ratio4_attention_replay as replay
+
+    attn = replay.synthetic_attention_block(DEV, hidden=256, n_heads=8, q_lora=64, index_heads=8, index_topk=16)
+
+    def make_cache(case, offset=30000):
+        return replay.make_seeded_cache(DEV, sliding_window=128, pooled_rows=case.pooled_rows, offset=offset)
+
+    gates = (dak._ENABLED, isk._ENABLED)
+    rep = replay.run_ratio4_attention_replay(attn, cache_cls=replay.SyntheticCache, make_cache=make_cache, hidden_size=256,
+                                             device=DEV, repeats=3, warmup=1, pooled_rows=[96, 12], index_topk=16,
+                                             stage_profile=True)
+    assert (dak._ENABLED, isk._ENABLED) == gates  # the gates are put back
+    assert rep["metric"] == "ds4_attention_one_layer_replay" and rep["input_tokens"] == 1
+    big, small = rep["cases"]
+    assert big["name"] == "ratio4_rows96_topk16" and big["median_seconds"] > 0 and big["min_seconds"] <= big["median_seconds"]
+    assert rep["fused_decode_calls"] == 4  # warm-up + repeats of the one engaged case
+    assert set(big["stages"]) >= {"decode_prep", "decode_sdpa", "partial_rope"}
+    assert big["stages"]["decode_prep"]["calls_per_layer_call"] == 1.0
+    assert big["stages"]["decode_sdpa"]["seconds_per_layer_call"] > 0
+    assert "skipped" in small  # a pool not larger than the selection belongs to the composed path
+    # the stage patch is gone: the module attributes are the plain functions again
+    assert dak.fused_decode_prep.__name__ == "fused_decode_prep"
+
+    rep = replay.run_ratio4_attention_replay(attn, cache_cls=replay.SyntheticCache,
+                                             make_cache=lambda case: make_cache(case, offset=0), hidden_size=256,
+                                             device=DEV, repeats=2, warmup=1, pooled_rows=[40], index_topk=16,
+                                             stage_profile=True, input_tokens=24)
+    (case,) = rep["cases"]
+    assert rep["prefill_fast_calls"] == 3 and case["median_seconds"] > 0
+    assert set(case["stages"]) >= {"prefill_attention", "prefill_scores", "prefill_q_qat", "topk", "partial_rope"}
+    assert case["stages"]["partial_rope"]["calls_per_layer_call"] == 4.0  # q, kv, indexer q, inverse on the output
