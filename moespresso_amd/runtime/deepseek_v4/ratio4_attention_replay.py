@@ -252,18 +252,20 @@ def make_seeded_cache(device, *, sliding_window: int, pooled_rows: int, head_dim
 
 # ---------------------------------------------------------------- replay
 
-def _time_case(layer: Callable[..., Any], make_cache: Callable[[Ratio4ReplayCase], Any], x: torch.Tensor,
-               case: Ratio4ReplayCase, *, repeats: int, warmup: int, profile: _StageProfile | None) -> dict[str, Any]:
+def _time_case(layer: Callable[..., Any], caches: list, x: torch.Tensor, case: Ratio4ReplayCase, *, repeats: int,
+               warmup: int, profile: _StageProfile | None) -> dict[str, Any]:
+    """``caches`` holds one fresh cache per call (warm-ups first): the ring append and the pool caches
+    start equal every time, and building them is not part of any timing."""
     mask = "causal" if int(x.shape[1]) > 1 else None
+    caches = list(caches)
     for _ in range(max(warmup, 0)):
-        layer(x, mask=mask, cache=make_cache(case))
+        layer(x, mask=mask, cache=caches.pop(0))
     torch.cuda.synchronize()
     if profile is not None:
         profile.reset()
     seconds = []
     for _ in range(repeats):
-        cache = make_cache(case)  # a fresh cache per call: the ring append and the pool caches start equal
-        torch.cuda.synchronize()
+        cache = caches.pop(0)
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
         layer(x, mask=mask, cache=cache)
@@ -319,11 +321,13 @@ def run_ratio4_attention_replay(attn: Any, *, cache_cls: type, make_cache: Calla
                                 "skipped": "served by the wrapped block's composed path"})
                 continue
             _set_index_topk(attn, case.index_topk)
+            caches = [make_cache(case) for _ in range(max(warmup, 0) + repeats)]
+            torch.cuda.synchronize()
             if profile is not None:
                 with _StagePatch(profile):
-                    results.append(_time_case(layer, make_cache, x, case, repeats=repeats, warmup=warmup, profile=profile))
+                    results.append(_time_case(layer, caches, x, case, repeats=repeats, warmup=warmup, profile=profile))
             else:
-                results.append(_time_case(layer, make_cache, x, case, repeats=repeats, warmup=warmup, profile=None))
+                results.append(_time_case(layer, caches, x, case, repeats=repeats, warmup=warmup, profile=None))
     finally:
         decode_attention_kernel._ENABLED, indexer_score_kernel._ENABLED = gates
     return {
