@@ -52,7 +52,7 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
   const int64_t n_tiles = (n_rows + 31) / 32;
   const int64_t stride = (int64_t)blocks_per_batch * 4;
   int64_t tile = (int64_t)blk * 4 + wave;
-  if (tile >= n_tiles) return;
+  const bool has_work = tile < n_tiles;  // a wave without a tile still brings its share of the query block
 
   // a tile image: the lane's 64 key bytes and the key's scale (loaded with the tile so that the wait
   // for it in the epilogue does not have to drain the tiles fetched behind it)
@@ -65,35 +65,53 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
     for (int j = 0; j < 4; j++) raw[j] = p[j];
   };
 
-  // the first two tiles go out before anything else: their HBM latency overlaps the query loads
+  // Prologue. The query block and the head weights are the same for every wave of the workgroup: each
+  // thread requests its share once (64 bytes of q, lanes of wave 0 one weight each), the first two
+  // tiles go out right behind, and while those fly the shares meet in LDS and every wave reads its
+  // A-operand registers back from there. (Every wave fetching all of q and its 32 weights itself kept
+  // the address units of a CU busy for about 3 us before the first tile could be multiplied.)
+  __shared__ __attribute__((aligned(16))) u32x4_t q_lds[2 * 8 * 64];  // [head tile][k-step][lane]: register images
+  __shared__ float w_lds[64];
+  u32x4_t qpiece[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int pc = tid + 256 * i;  // piece (head h, 8-column group c)
+    const int h = pc >> 4, c = pc & 15;
+    qpiece[i] = *reinterpret_cast<const u32x4_t*>(qb + (int64_t)(h < n_heads ? h : 0) * 128 + c * 8);
+  }
+  float wmine = wb[lane < n_heads ? lane : 0];
   u32x4_t ra[4], rb[4], rc[4];
   float sa, sb_, sc;
   const int64_t last = n_tiles - 1;
-  load_tile(tile, ra, sa);
+  load_tile(has_work ? tile : last, ra, sa);
   load_tile(tile + stride < n_tiles ? tile + stride : last, rb, sb_);
+  // (pinned here: the waits for the shares then leave the tile loads in flight, and the compiler cannot
+  // sink the share loads into the conditional stores below, behind the tile loads)
+#pragma unroll
+  for (int i = 0; i < 4; i++) asm volatile("" : "+v"(qpiece[i]));
+  asm volatile("" : "+v"(wmine));
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int pc = tid + 256 * i;
+    const int h = pc >> 4, c = pc & 15;
+    // slot of lane (m = h % 32, g = c / 8) in the image of (head tile h / 32, k-step c % 8)
+    q_lds[((h >> 5) * 8 + (c & 7)) * 64 + 32 * (c >> 3) + (h & 31)] = h < n_heads ? qpiece[i] : u32x4_t{0u, 0u, 0u, 0u};
+  }
+  if (wave == 0) w_lds[lane] = lane < n_heads ? wmine : 0.0f;
+  __syncthreads();
+  if (!has_work) return;
   // A operand: lane (m -> head, g) holds q[head][64g + 8s .. +7] for k-step s; heads past the end are zero
   u32x4_t qa[2][8];
 #pragma unroll
-  for (int mt = 0; mt < 2; mt++) {
-    const int head = 32 * mt + m;
-    const bool live = head < n_heads;
-    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(qb + (int64_t)(live ? head : 0) * 128 + 64 * g);
-    u32x4_t raw[8];
+  for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-    for (int s = 0; s < 8; s++) raw[s] = p[s];  // unconditional (clamped) loads, selected afterwards
-#pragma unroll
-    for (int s = 0; s < 8; s++) qa[mt][s] = live ? raw[s] : u32x4_t{0u, 0u, 0u, 0u};
-  }
+    for (int s = 0; s < 8; s++) qa[mt][s] = q_lds[(mt * 8 + s) * 64 + lane];
   // weights of this lane's accumulator rows: head = 32mt + 8(i/4) + 4g + i%4
   float wl[2][16];
 #pragma unroll
   for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const int head = 32 * mt + 8 * (i / 4) + 4 * g + (i % 4);
-      const float wv = wb[head < n_heads ? head : 0];
-      wl[mt][i] = head < n_heads ? wv : 0.0f;
-    }
+    for (int i = 0; i < 16; i++) wl[mt][i] = w_lds[32 * mt + 8 * (i / 4) + 4 * g + (i % 4)];
 
   auto compute_tile = [&](int64_t t, const u32x4_t (&cur)[4], float ks) {
     const int64_t row = t * 32 + m;
