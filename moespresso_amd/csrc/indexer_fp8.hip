@@ -29,6 +29,11 @@ __device__ __forceinline__ float relu_bits(float x) {
   return __int_as_float(v > 0 ? v : 0);
 }
 
+// PAIRS: a wave takes its keys in units of two consecutive 32-key tiles, so that the key scales come in
+// and the scores go out 64 rows (256 bytes) at a time, one row per lane; a per-tile 128-byte load and
+// store each cost a DRAM page of their own for 3 % of the bytes and measurably more of the time. The
+// single-tile form spreads short rows and small batches over more waves.
+template <bool PAIRS>
 __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16_t* __restrict__ q,
                                                                     const uint8_t* __restrict__ keys,
                                                                     const float* __restrict__ key_scales,
@@ -49,10 +54,11 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
   const float* wb = weights + (int64_t)b * n_heads;
   float* sb = scores + (int64_t)b * n_rows;
 
-  const int64_t n_tiles = (n_rows + 31) / 32;
+  // work items: tiles, or units of two tiles
+  const int64_t n_tiles = PAIRS ? (n_rows + 63) / 64 : (n_rows + 31) / 32;
   const int64_t stride = (int64_t)blocks_per_batch * 4;
   int64_t tile = (int64_t)blk * 4 + wave;
-  const bool has_work = tile < n_tiles;  // a wave without a tile still brings its share of the query block
+  const bool has_work = tile < n_tiles;  // a wave without work still brings its share of the query block
 
   // a tile image: the lane's 64 key bytes and the key's scale (loaded with the tile so that the wait
   // for it in the epilogue does not have to drain the tiles fetched behind it)
@@ -63,6 +69,19 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
     const u32x4_t* p = reinterpret_cast<const u32x4_t*>(kb + row * 128 + 64 * g);
 #pragma unroll
     for (int j = 0; j < 4; j++) raw[j] = p[j];
+  };
+  // half h of unit u: rows [64 u + 32 h, +32); the unit's 64 scales, one per lane, travel with half 0
+  auto load_half = [&](int64_t u, int h, u32x4_t (&raw)[4]) {
+    int64_t row = u * 64 + 32 * h + m;
+    if (row >= n_rows) row = n_rows - 1;
+    const u32x4_t* p = reinterpret_cast<const u32x4_t*>(kb + row * 128 + 64 * g);
+#pragma unroll
+    for (int j = 0; j < 4; j++) raw[j] = p[j];
+  };
+  auto load_unit_scales = [&](int64_t u) -> float {
+    int64_t row = u * 64 + lane;
+    if (row >= n_rows) row = n_rows - 1;
+    return ksb[row];
   };
 
   // Prologue. The query block and the head weights are the same for every wave of the workgroup: each
@@ -80,11 +99,18 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
     qpiece[i] = *reinterpret_cast<const u32x4_t*>(qb + (int64_t)(h < n_heads ? h : 0) * 128 + c * 8);
   }
   float wmine = wb[lane < n_heads ? lane : 0];
-  u32x4_t ra[4], rb[4], rc[4];
+  u32x4_t ra[4], rb[4], rc[4], rd[4];
   float sa, sb_, sc;
   const int64_t last = n_tiles - 1;
-  load_tile(has_work ? tile : last, ra, sa);
-  load_tile(tile + stride < n_tiles ? tile + stride : last, rb, sb_);
+  if constexpr (PAIRS) {
+    const int64_t u0 = has_work ? tile : last;
+    sa = load_unit_scales(u0);
+    load_half(u0, 0, ra);
+    load_half(u0, 1, rb);
+  } else {
+    load_tile(has_work ? tile : last, ra, sa);
+    load_tile(tile + stride < n_tiles ? tile + stride : last, rb, sb_);
+  }
   // (pinned here: the waits for the shares then leave the tile loads in flight, and the compiler cannot
   // sink the share loads into the conditional stores below, behind the tile loads)
 #pragma unroll
@@ -113,8 +139,8 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
 #pragma unroll
     for (int i = 0; i < 16; i++) wl[mt][i] = w_lds[32 * mt + 8 * (i / 4) + 4 * g + (i % 4)];
 
-  auto compute_tile = [&](int64_t t, const u32x4_t (&cur)[4], float ks) {
-    const int64_t row = t * 32 + m;
+  // relu-weighted head sum of the 32 keys of one tile image: lane (m, either g) gets the sum of key m
+  auto tile_sums = [&](const u32x4_t (&cur)[4]) -> float {
     f32x16_t acc0 = {0}, acc1 = {0};
 #pragma unroll
     for (int s = 0; s < 8; s++) {
@@ -132,9 +158,42 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
 #pragma unroll
     for (int i = 0; i < 16; i++) sum = fmaf(relu_bits(acc1[i]), wl[1][i], sum);
     sum += __shfl_xor(sum, 32, MSPR_WAVE);
+    return sum;
+  };
+  auto compute_tile = [&](int64_t t, const u32x4_t (&cur)[4], float ks) {
+    const int64_t row = t * 32 + m;
+    const float sum = tile_sums(cur);
     if (g == 0 && row < n_rows) sb[row] = sum * ks;
   };
+  // both halves of a unit, then one 64-lane store: lane (m, g) holds row 64 u + 32 g + m
+  auto compute_unit = [&](int64_t u, const u32x4_t (&h0)[4], const u32x4_t (&h1)[4], float ks_lane) {
+    const float s0 = tile_sums(h0);
+    const float s1 = tile_sums(h1);
+    const int64_t row = u * 64 + lane;
+    if (row < n_rows) sb[row] = (g ? s1 : s0) * ks_lane;
+  };
 
+  if constexpr (PAIRS) {
+    // Two units' images alternate: while a unit is multiplied the next one (8 KB) is in flight. Loads past
+    // the wave's last unit are clamped re-reads and are never consumed.
+    while (true) {
+      int64_t nu = tile + stride < n_tiles ? tile + stride : last;
+      sb_ = load_unit_scales(nu);
+      load_half(nu, 0, rc);
+      load_half(nu, 1, rd);
+      compute_unit(tile, ra, rb, sa);
+      tile += stride;
+      if (tile >= n_tiles) break;
+      nu = tile + stride < n_tiles ? tile + stride : last;
+      sa = load_unit_scales(nu);
+      load_half(nu, 0, ra);
+      load_half(nu, 1, rb);
+      compute_unit(tile, rc, rd, sb_);
+      tile += stride;
+      if (tile >= n_tiles) break;
+    }
+    return;
+  }
   // Three tile images rotate through registers: while one is multiplied the next two are in flight
   // (8 KB per wave). Loads past the wave's last tile are clamped re-reads and are never consumed.
   while (true) {
@@ -157,8 +216,10 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
 
 int mspr_launch_indexer_scores_fp8(const void* q, const void* keys, const float* key_scales, const float* weights,
                                    int batch, int n_heads, int64_t n_rows, float* scores, hipStream_t st) {
-  const int64_t n_tiles = (n_rows + 31) / 32;
-  // about 2 workgroups per CU in total, every wave with at least one tile
+  // units of two tiles once every wave of a full grid (2 workgroups per CU) still gets at least two of them
+  const bool pairs = (int64_t)batch * ((n_rows + 63) / 64) >= 2 * 2048;
+  const int64_t n_tiles = pairs ? (n_rows + 63) / 64 : (n_rows + 31) / 32;
+  // about 2 workgroups per CU in total, every wave with at least one work item
   int64_t per_batch = (512 + batch - 1) / batch;
   int64_t max_blocks = (n_tiles + 3) / 4;
   if (per_batch > max_blocks) per_batch = max_blocks;
@@ -166,9 +227,14 @@ int mspr_launch_indexer_scores_fp8(const void* q, const void* keys, const float*
   dim3 grid((unsigned)(per_batch * batch)), block(256);
   {
     MsprProfScope prof(MSPR_K_INDEXER_FP8, st);
-    indexer_scores_fp8_kernel<<<grid, block, 0, st>>>(reinterpret_cast<const uint16_t*>(q),
-                                                       reinterpret_cast<const uint8_t*>(keys), key_scales, weights,
-                                                       n_heads, n_rows, (int)per_batch, scores);
+    if (pairs)
+      indexer_scores_fp8_kernel<true><<<grid, block, 0, st>>>(reinterpret_cast<const uint16_t*>(q),
+                                                               reinterpret_cast<const uint8_t*>(keys), key_scales, weights,
+                                                               n_heads, n_rows, (int)per_batch, scores);
+    else
+      indexer_scores_fp8_kernel<false><<<grid, block, 0, st>>>(reinterpret_cast<const uint16_t*>(q),
+                                                                reinterpret_cast<const uint8_t*>(keys), key_scales, weights,
+                                                                n_heads, n_rows, (int)per_batch, scores);
   }
   MSPR_CHECK_LAUNCH("indexer_scores_fp8");
   return MSPR_OK;

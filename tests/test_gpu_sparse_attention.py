@@ -169,8 +169,11 @@ def test_sparse_mla_decode_full_config_batch16_with_sinks():
     assert err < 2e-3, err
 
 
+# (the last three take the two-tiles-per-unit form of the kernel: an odd tile count, a ragged last tile,
+# a ragged first half of the last unit)
 @pytest.mark.parametrize("cfg", [dict(B=1, H=64, N=1000), dict(B=3, H=64, N=4099), dict(B=2, H=20, N=64),
-                                 dict(B=16, H=64, N=32768)])
+                                 dict(B=16, H=64, N=32768), dict(B=16, H=64, N=16416), dict(B=20, H=33, N=13123),
+                                 dict(B=32, H=64, N=8209)])
 def test_indexer_scores_fp8_and_topk(cfg):
     B, H, N = cfg["B"], cfg["H"], cfg["N"]
     rng = np.random.default_rng(B * 1000 + N)
