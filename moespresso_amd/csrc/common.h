@@ -88,6 +88,32 @@ __device__ __forceinline__ float load_as_f32(const void* p, int64_t i) {
 
 __device__ __forceinline__ float wave_xor_f32(float v, int mask) { return __shfl_xor(v, mask, MSPR_WAVE); }
 
+// The value lane (l ^ M) holds, for a single-bit M. Inside a row of 16 lanes the exchange is one or two
+// data-parallel-primitive moves (quad permutes give l^1, l^2, l^3; the half-row and row mirrors give
+// l^7 and l^15, and two of them compose to l^4 and l^8), which cost an ALU slot and no LDS round trip;
+// l^16 is a bit-mask swizzle, l^32 the general lane permute.
+template <int M>
+__device__ __forceinline__ float lane_xor(float v) {
+  static_assert(M == 1 || M == 2 || M == 4 || M == 8 || M == 16 || M == 32, "single-bit lane masks only");
+  int x = __float_as_int(v);
+  if constexpr (M == 1) {
+    x = __builtin_amdgcn_mov_dpp(x, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  } else if constexpr (M == 2) {
+    x = __builtin_amdgcn_mov_dpp(x, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  } else if constexpr (M == 4) {
+    x = __builtin_amdgcn_mov_dpp(x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l^7
+    x = __builtin_amdgcn_mov_dpp(x, 0x1B, 0xF, 0xF, true);   // quad_perm [3,2,1,0]: l^3
+  } else if constexpr (M == 8) {
+    x = __builtin_amdgcn_mov_dpp(x, 0x140, 0xF, 0xF, true);  // row_mirror: l^15
+    x = __builtin_amdgcn_mov_dpp(x, 0x141, 0xF, 0xF, true);  // row_half_mirror: l^7
+  } else if constexpr (M == 16) {
+    x = __builtin_amdgcn_ds_swizzle(x, 0x401F);  // and 0x1F, or 0, xor 0x10
+  } else {
+    x = __shfl_xor(x, 32, MSPR_WAVE);
+  }
+  return __int_as_float(x);
+}
+
 // Monotone float32 -> uint32 map: negatives inverted, positives offset. Orders -0.0 below +0.0
 // and +NaN above +inf.
 __device__ __forceinline__ uint32_t score_key(float s) {
@@ -104,7 +130,8 @@ __device__ __forceinline__ uint32_t score_key(float s) {
 // g_pow2_tab holds float32(exp(float32(k*ln2f))) for k = -160..160. Away from powers of two the
 // ceil is decided from the exponent field; within 2^-12 of one (and for non-finite or zero input)
 // a float64 log decides it, which rounds to the same float32 value the table path assumes.
-__device__ __forceinline__ float pow2_group_scale(float amax, float denom) {
+// `tab` may be a copy of the table in LDS.
+__device__ __forceinline__ float pow2_group_scale(float amax, float denom, const float* tab = g_pow2_tab) {
   float r = amax / denom;
   uint32_t u = __float_as_uint(r);
   uint32_t ex = (u >> 23) & 0xFFu;
@@ -112,7 +139,7 @@ __device__ __forceinline__ float pow2_group_scale(float amax, float denom) {
   bool fast = (u >> 31) == 0u && ex != 0u && ex != 0xFFu && man > 0x800u && man < 0x7FF800u;
   if (fast) {
     int k = (int)ex - 127 + 1;
-    return g_pow2_tab[k - MSPR_POW2_TAB_MIN];
+    return tab[k - MSPR_POW2_TAB_MIN];
   }
   float l = (float)log((double)r);
   float l2 = l / MSPR_LN2F;

@@ -19,8 +19,9 @@ extern "C" int mspr_fused_decode_prep(const void* q_idx, int q_dtype, int n_head
   MSPR_REQUIRE(q_dtype >= MSPR_F32 && q_dtype <= MSPR_BF16, "fused_decode_prep: q_idx must be f32, f16 or bf16");
   MSPR_REQUIRE(n_rows >= 1 && n_rows < (int64_t)1 << 31, "fused_decode_prep: n_rows out of range");
   MSPR_REQUIRE(topk > 0 && topk < n_rows, "fused_decode_prep: topk must be positive and smaller than n_rows");
-  MSPR_REQUIRE(mspr_aligned(q_idx, 16) && mspr_aligned(pooled_qat, 16),
-               "fused_decode_prep: q_idx and pooled_qat must be 16-byte aligned");
+  MSPR_REQUIRE(mspr_aligned(q_idx, 16) && mspr_aligned(pooled_qat, 16) && mspr_aligned(kv_row, 16) &&
+                   mspr_aligned(row_out, 16),
+               "fused_decode_prep: q_idx, pooled_qat, kv_row and row_out must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   int rc = mspr_launch_scores_f32(q_idx, q_dtype, n_heads, pooled_qat, n_rows, weights, scale, scores, true, st);
   if (rc != MSPR_OK) return rc;

@@ -2,10 +2,11 @@
 // E4M3FN row round trip and the prepared KV row of the fused decode island.
 //
 // Layout notes (wave64): one 128-wide row lives in one half-wave, four elements per lane, so the
-// Hadamard butterflies of strides 4..64 are xor shuffles inside the half. The score row runs on
-// the float32 MFMA (32x32x2): heads are the M dimension, pool rows the N dimension, so the
-// per-row head sum stays inside a lane (plus one xor-32 shuffle) and pool rows stream from HBM
-// straight into the B operand registers, 256 contiguous bytes per lane.
+// Hadamard butterflies of strides 4..64 are lane exchanges inside the half (data-parallel-primitive
+// moves up to stride 32, one swizzle for stride 64). The score row runs on the bf16 MFMA (32x32x16)
+// with exact products: heads are the M dimension, pool rows the N dimension, so the per-row head sum
+// stays inside a lane (plus one xor-32 shuffle) and pool rows stream from HBM straight into the B
+// operand registers, 256 contiguous bytes per lane.
 #include "common.h"
 #include "profile.h"
 
@@ -23,6 +24,7 @@ __device__ __forceinline__ float add_rn(float a, float b) { return a + b; }
 constexpr float kHadamardScale = 0.08838834764831845f;  // float32(128^-1/2)
 constexpr float kAmaxFloor = 7.052966104933725e-38f;      // 6 * 2^-126
 constexpr float kFp8AmaxFloor = 1.0e-4f;
+constexpr int kPow2TabLen = 321;  // entries of g_pow2_tab
 
 // MLX Maximum(x, floor): NaN passes through.
 __device__ __forceinline__ float mx_floor_max(float x, float fl) { return isnan(x) ? x : (x > fl ? x : fl); }
@@ -33,69 +35,93 @@ __device__ __forceinline__ float mx_floor_max(float x, float fl) { return isnan(
 // nearest lattice value.
 // LIVE selects the prefill-side variant (indexed_attention_kernel.py:1125-1202 of the reference):
 // scale 2^ceil(log2(amax/6)) taken exactly, ties to the even lattice index.
-template <bool LIVE = false>
-__device__ __forceinline__ f32x4_t qat128(f32x4_t v, int lane32) {
+// First half: the butterflies, the 128^-1/2 scale and the floored amax of this lane's group of 32.
+struct QatRotated {
+  f32x4_t x;
+  float amax;
+};
+
+// One cross-lane butterfly stage: lanes with bit M clear take x + o, the others o - x, where o is the
+// partner lane's value. Written as fma(x, +-1, o): the product is exact, so the single rounding is that
+// of the sum or difference itself.
+template <int M>
+__device__ __forceinline__ f32x4_t butterfly_stage(f32x4_t x, int lane32) {
+  const float sgn = (lane32 & M) ? -1.0f : 1.0f;
+  return f32x4_t{__builtin_fmaf(x.x, sgn, lane_xor<M>(x.x)), __builtin_fmaf(x.y, sgn, lane_xor<M>(x.y)),
+                 __builtin_fmaf(x.z, sgn, lane_xor<M>(x.z)), __builtin_fmaf(x.w, sgn, lane_xor<M>(x.w))};
+}
+
+template <int M>
+__device__ __forceinline__ float amax_stage(float amax) {
+  const float o = lane_xor<M>(amax);
+  return (isnan(amax) || isnan(o)) ? __builtin_nanf("") : fmaxf(amax, o);
+}
+
+__device__ __forceinline__ QatRotated qat_rotate(f32x4_t v, int lane32) {
   float a0 = v.x + v.y, a1 = v.x - v.y, a2 = v.z + v.w, a3 = v.z - v.w;
   f32x4_t x = {a0 + a2, a1 + a3, a0 - a2, a1 - a3};
-#pragma unroll
-  for (int m = 1; m <= 16; m <<= 1) {
-    f32x4_t o;
-    o.x = __shfl_xor(x.x, m, MSPR_WAVE);
-    o.y = __shfl_xor(x.y, m, MSPR_WAVE);
-    o.z = __shfl_xor(x.z, m, MSPR_WAVE);
-    o.w = __shfl_xor(x.w, m, MSPR_WAVE);
-    x = (lane32 & m) ? (o - x) : (x + o);
-  }
+  x = butterfly_stage<1>(x, lane32);
+  x = butterfly_stage<2>(x, lane32);
+  x = butterfly_stage<4>(x, lane32);
+  x = butterfly_stage<8>(x, lane32);
+  x = butterfly_stage<16>(x, lane32);
   x = x * kHadamardScale;
   // fmaxf drops NaN operands; carry NaN explicitly so a NaN element poisons its group
   bool any_nan = isnan(x.x) || isnan(x.y) || isnan(x.z) || isnan(x.w);
   float amax = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
   if (any_nan) amax = __builtin_nanf("");
-#pragma unroll
-  for (int m = 1; m <= 4; m <<= 1) {
-    float o = __shfl_xor(amax, m, MSPR_WAVE);
-    amax = (isnan(amax) || isnan(o)) ? __builtin_nanf("") : fmaxf(amax, o);
-  }
-  amax = mx_floor_max(amax, kAmaxFloor);
-  float scale;
+  amax = amax_stage<1>(amax);
+  amax = amax_stage<2>(amax);
+  amax = amax_stage<4>(amax);
+  return QatRotated{x, mx_floor_max(amax, kAmaxFloor)};
+}
+
+template <bool LIVE = false>
+__device__ __forceinline__ float qat_scale(float amax, const float* tab = g_pow2_tab) {
   if constexpr (LIVE) {
     const float r = amax / 6.0f;
-    const uint32_t u = __float_as_uint(r);
-    if (isnan(r) || isinf(r)) {
-      scale = r;
-    } else {
-      int e;
-      const float m = frexpf(r, &e);  // r = m * 2^e, m in [0.5, 1)
-      scale = ldexpf(1.0f, m == 0.5f ? e - 1 : e);
-    }
-    (void)u;
+    if (isnan(r) || isinf(r)) return r;
+    int e;
+    const float m = frexpf(r, &e);  // r = m * 2^e, m in [0.5, 1)
+    return ldexpf(1.0f, m == 0.5f ? e - 1 : e);
   } else {
-    scale = pow2_group_scale(amax, 6.0f);
+    return pow2_group_scale(amax, 6.0f, tab);
   }
-  const float lattice[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+}
+
+// Second half: clip to [-6, 6] in units of the scale and take the nearest lattice value
+// {0, .5, 1, 1.5, 2, 3, 4, 6}. The reference takes the first minimum of |n - lattice[k]|; around a
+// midpoint of two neighbours both differences are exact float32 values (each operand is within a factor
+// of two of the other, or the lattice value is 0), so comparing |n| with the midpoints picks the same
+// value, ties going to the lower neighbour. The LIVE variant breaks ties towards the even lattice index,
+// which turns three of the seven comparisons into >=. NaN compares false everywhere and lands on 0.
+template <bool LIVE = false>
+__device__ __forceinline__ f32x4_t qat_snap(f32x4_t x, float scale) {
   f32x4_t out;
 #pragma unroll
   for (int j = 0; j < 4; j++) {
     float n = x[j] / scale;
     n = (isnan(n) || n > -6.0f) ? n : -6.0f;
     n = (isnan(n) || n < 6.0f) ? n : 6.0f;
-    float absn = fabsf(n);
-    float best = fabsf(absn - lattice[0]);
-    float dq = lattice[0];
-    bool best_odd = false;
-#pragma unroll
-    for (int k = 1; k < 8; k++) {
-      float d = fabsf(absn - lattice[k]);
-      if (d < best || (LIVE && d == best && (k & 1) == 0 && best_odd)) {
-        best = d;
-        dq = lattice[k];
-        best_odd = (k & 1) != 0;
-      }
-    }
+    const float a = fabsf(n);
+    float dq = 0.0f;
+    dq = a > 0.25f ? 0.5f : dq;
+    dq = (LIVE ? a >= 0.75f : a > 0.75f) ? 1.0f : dq;
+    dq = a > 1.25f ? 1.5f : dq;
+    dq = (LIVE ? a >= 1.75f : a > 1.75f) ? 2.0f : dq;
+    dq = a > 2.5f ? 3.0f : dq;
+    dq = (LIVE ? a >= 3.5f : a > 3.5f) ? 4.0f : dq;
+    dq = a > 5.0f ? 6.0f : dq;
     dq = n < 0.0f ? -dq : dq;
     out[j] = dq * scale;
   }
   return out;
+}
+
+template <bool LIVE = false>
+__device__ __forceinline__ f32x4_t qat128(f32x4_t v, int lane32) {
+  const QatRotated r = qat_rotate(v, lane32);
+  return qat_snap<LIVE>(r.x, qat_scale<LIVE>(r.amax));
 }
 
 template <int DT>
@@ -130,53 +156,122 @@ __global__ __launch_bounds__(256) void qat_rows_kernel(const void* __restrict__ 
 }
 
 // ------------------------------------------------------------------ score row, float32 pool rows
-// Block = 4 waves. The block QATs the (up to 64) query heads into LDS once, each wave then keeps
-// them in registers as the MFMA A operand and walks 32-row tiles of the pool.
+// Block = 8 waves. The block QATs the (up to 64) query heads into LDS once (four rows per lane, while
+// the wave's first pool tile is already on its way), each wave then keeps them in registers as the
+// MFMA A operand and walks 32-row tiles of the pool.
+//
+// The contraction runs on the bf16 MFMA (32x32x16) without giving up exact products: a QAT'd query
+// value is a lattice value times a power of two (three significant bits), so it is a bf16 number, and
+// so is a QAT'd pool value. A pool tile whose 32-bit words all have a zero low half is multiplied as
+// it is (one bf16 piece per value); any other tile is split into three bf16 pieces per value
+// (truncated high part, truncated remainder, rest: 8 + 8 + 8 significant bits, exact) and takes three
+// passes. Products of two bf16 numbers are exact in the float32 accumulator either way. The float32
+// MFMA (32x32x2) this replaces needed 128 instructions of 16 passes per tile against 16 of 8.
+__device__ __forceinline__ uint32_t pack_hi16(float lo, float hi) {
+  // the high halves of two float32 words side by side: two bf16 values by truncation
+  return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+
+constexpr int kScoreThreads = 512;
+constexpr int kScoreWaves = kScoreThreads / 64;
+// float32 row pitch of the QAT'd query block in LDS: 128 values plus 4, so that the 16-byte reads of
+// 16 lanes holding 16 different heads fall into different banks
+constexpr int kQPitch = 132;
+
 template <int DT, bool STAGE_HALF>
-__global__ __launch_bounds__(256) void scores_f32_kernel(const void* __restrict__ q, int n_heads,
-                                                         const float* __restrict__ pooled, int64_t n_rows,
-                                                         const float* __restrict__ weights, float scale,
-                                                         float* __restrict__ scores) {
-  __shared__ float qbuf[64 * 128];
+__global__ __launch_bounds__(kScoreThreads) void scores_f32_kernel(const void* __restrict__ q, int n_heads,
+                                                                   const float* __restrict__ pooled, int64_t n_rows,
+                                                                   const float* __restrict__ weights, float scale,
+                                                                   float* __restrict__ scores) {
+  __shared__ float qbuf[64 * kQPitch];
   __shared__ float wbuf[64];
+  __shared__ float ptab[kPow2TabLen];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int lane32 = tid & 31;
   const int wave = tid >> 6;
   const int half = (tid >> 5) & 1;
+  const int m = lane & 31;
+  const int g = lane >> 5;
 
-  // QAT pass: 8 rows per step (two per wave)
-  for (int h0 = 0; h0 < 64; h0 += 8) {
-    int h = h0 + wave * 2 + half;
-    int src = h < n_heads ? h : n_heads - 1;
-    f32x4_t v = load_row4<DT>(q, src, lane32);
-    f32x4_t y = qat128(v, lane32);
+  const int64_t n_tiles = (n_rows + 31) / 32;
+  const int64_t wave_stride = (int64_t)gridDim.x * kScoreWaves;
+  int64_t tile = (int64_t)blockIdx.x * kScoreWaves + wave;
+
+  // The eight waves QAT the 64 query rows, one row per half-wave and four rows per lane; the rows of a
+  // lane are fetched together and the power-of-two table sits in LDS, so the pass waits for memory once.
+  f32x4_t raw[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int h = 16 * i + wave * 2 + half;
+    raw[i] = load_row4<DT>(q, h < n_heads ? h : n_heads - 1, lane32);
+  }
+  const float tab_a = g_pow2_tab[tid < kPow2TabLen ? tid : 0];
+  const float w_mine = weights[tid < n_heads ? tid : 0];
+  // The first pool tile of the wave is requested now and lands while the queries are prepared. Lane
+  // (m = row, g) owns the 64 consecutive float32 values [64 g, 64 g + 64) of its pool row.
+  float kv[64];
+  auto load_tile = [&](int64_t t) {
+    int64_t src = t * 32 + m;
+    src = src < n_rows ? src : n_rows - 1;
+    const f32x4_t* kp = reinterpret_cast<const f32x4_t*>(pooled + src * 128 + 64 * g);
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+      const f32x4_t t4 = kp[j];
+      kv[4 * j] = t4.x;
+      kv[4 * j + 1] = t4.y;
+      kv[4 * j + 2] = t4.z;
+      kv[4 * j + 3] = t4.w;
+    }
+  };
+  load_tile(tile < n_tiles ? tile : n_tiles - 1);
+
+  if (tid < kPow2TabLen) ptab[tid] = tab_a;
+  if (tid < 64) wbuf[tid] = tid < n_heads ? w_mine : 0.0f;
+  __syncthreads();
+  QatRotated rot[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) rot[i] = qat_rotate(raw[i], lane32);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int h = 16 * i + wave * 2 + half;
+    f32x4_t y = qat_snap(rot[i].x, qat_scale(rot[i].amax, ptab));
     if (STAGE_HALF) {
 #pragma unroll
       for (int j = 0; j < 4; j++) y[j] = f16_bits_to_f32(f32_to_f16_bits(y[j]));
     }
     if (h >= n_heads) y = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    reinterpret_cast<f32x4_t*>(qbuf + h * 128)[lane32] = y;
+    reinterpret_cast<f32x4_t*>(qbuf + h * kQPitch)[lane32] = y;
   }
-  if (tid < 64) wbuf[tid] = tid < n_heads ? weights[tid] : 0.0f;
   __syncthreads();
 
-  // A operand: lane (m = lane%32 -> head, g = lane/32) supplies q[head][64g + s] at k-step s
-  const int m = lane & 31;
-  const int g = lane >> 5;
-  float qa[2][64];
+  // A operand: lane (m -> head, g) holds q[head][64 g + 8 s .. + 7] as bf16 for k-step s. Piece 0 is the
+  // truncated value itself (all of it for a bf16 number), pieces 1 and 2 the truncated remainders.
+  auto q_piece = [&](int mt, int s, int piece) -> u32x4_t {
+    const f32x4_t t0 = *reinterpret_cast<const f32x4_t*>(qbuf + (mt * 32 + m) * kQPitch + 64 * g + 8 * s);
+    const f32x4_t t1 = *reinterpret_cast<const f32x4_t*>(qbuf + (mt * 32 + m) * kQPitch + 64 * g + 8 * s + 4);
+    float v[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+    for (int p = 0; p < piece; p++)
+#pragma unroll
+      for (int j = 0; j < 8; j++) v[j] = v[j] - __uint_as_float(__float_as_uint(v[j]) & 0xFFFF0000u);
+    return u32x4_t{pack_hi16(v[0], v[1]), pack_hi16(v[2], v[3]), pack_hi16(v[4], v[5]), pack_hi16(v[6], v[7])};
+  };
+  u32x4_t qa[2][8];
+  uint32_t q_low = 0u;
 #pragma unroll
   for (int mt = 0; mt < 2; mt++) {
 #pragma unroll
-    for (int s = 0; s < 64; s += 4) {
-      // rotate the column by the row to spread LDS banks
-      f32x4_t t = *reinterpret_cast<const f32x4_t*>(qbuf + (mt * 32 + m) * 128 + 64 * g + s);
-      qa[mt][s] = t.x;
-      qa[mt][s + 1] = t.y;
-      qa[mt][s + 2] = t.z;
-      qa[mt][s + 3] = t.w;
+    for (int s = 0; s < 8; s++) {
+      const u32x4_t* src = reinterpret_cast<const u32x4_t*>(qbuf + (mt * 32 + m) * kQPitch + 64 * g + 8 * s);
+      const u32x4_t t0 = src[0], t1 = src[1];
+      qa[mt][s] = u32x4_t{__builtin_amdgcn_perm(t0.y, t0.x, 0x07060302u), __builtin_amdgcn_perm(t0.w, t0.z, 0x07060302u),
+                          __builtin_amdgcn_perm(t1.y, t1.x, 0x07060302u), __builtin_amdgcn_perm(t1.w, t1.z, 0x07060302u)};
+      q_low |= t0.x | t0.y | t0.z | t0.w | t1.x | t1.y | t1.z | t1.w;
     }
   }
+  // a QAT'd value is a bf16 number (zero low half) unless the input was out of range; then the whole
+  // workgroup takes the three-piece form (the pieces come from LDS again, they are not kept in registers)
+  const bool q_exact = __syncthreads_and((q_low & 0xFFFFu) == 0u);
   // head weights for this lane's accumulator rows: head = 32mt + 8(i/4) + 4g + i%4
   float wl[2][16];
 #pragma unroll
@@ -184,28 +279,50 @@ __global__ __launch_bounds__(256) void scores_f32_kernel(const void* __restrict_
 #pragma unroll
     for (int i = 0; i < 16; i++) wl[mt][i] = wbuf[32 * mt + 8 * (i / 4) + 4 * g + (i % 4)];
 
-  const int64_t n_tiles = (n_rows + 31) / 32;
-  const int64_t wave_global = (int64_t)blockIdx.x * 4 + wave;
-  const int64_t wave_stride = (int64_t)gridDim.x * 4;
-  for (int64_t tile = wave_global; tile < n_tiles; tile += wave_stride) {
-    int64_t row = tile * 32 + m;
-    int64_t src = row < n_rows ? row : n_rows - 1;
-    const f32x4_t* kp = reinterpret_cast<const f32x4_t*>(pooled + src * 128 + 64 * g);
-    float kb[64];
+  while (tile < n_tiles) {
+    const int64_t row = tile * 32 + m;
+    uint32_t low = 0u;
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
-      f32x4_t t = kp[j];
-      kb[4 * j] = t.x;
-      kb[4 * j + 1] = t.y;
-      kb[4 * j + 2] = t.z;
-      kb[4 * j + 3] = t.w;
-    }
+    for (int j = 0; j < 64; j++) low |= __float_as_uint(kv[j]);
+    const bool k_exact = __all((low & 0xFFFFu) == 0u);  // wave-uniform
     f32x16_t acc0 = {0}, acc1 = {0};
+    auto k_operand = [&](const float (&kk)[64], int s) -> bf16x8_t {
+      const u32x4_t kf = {pack_hi16(kk[8 * s], kk[8 * s + 1]), pack_hi16(kk[8 * s + 2], kk[8 * s + 3]),
+                          pack_hi16(kk[8 * s + 4], kk[8 * s + 5]), pack_hi16(kk[8 * s + 6], kk[8 * s + 7])};
+      return __builtin_bit_cast(bf16x8_t, kf);
+    };
+    if (k_exact && q_exact) {
 #pragma unroll
-    for (int s = 0; s < 64; s++) {
-      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[0][s], kb[s], acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[1][s], kb[s], acc1, 0, 0, 0);
+      for (int s = 0; s < 8; s++) {
+        const bf16x8_t kfb = k_operand(kv, s);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, qa[0][s]), kfb, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, qa[1][s]), kfb, acc1, 0, 0, 0);
+      }
+    } else {
+      // every piece of q meets every piece of k, smallest products first
+      const int q_pieces = q_exact ? 1 : 3;
+      for (int kp_i = 2; kp_i >= 0; kp_i--) {
+        float kk[64];
+#pragma unroll
+        for (int j = 0; j < 64; j++) {
+          float v = kv[j];
+          for (int p = 0; p < kp_i; p++) v = v - __uint_as_float(__float_as_uint(v) & 0xFFFF0000u);
+          kk[j] = v;
+        }
+        for (int qp_i = q_pieces - 1; qp_i >= 0; qp_i--) {
+#pragma unroll
+          for (int s = 0; s < 8; s++) {
+            const bf16x8_t kfb = k_operand(kk, s);
+            const u32x4_t q0 = qp_i == 0 ? qa[0][s] : q_piece(0, s, qp_i);
+            const u32x4_t q1 = qp_i == 0 ? qa[1][s] : q_piece(1, s, qp_i);
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, q0), kfb, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, q1), kfb, acc1, 0, 0, 0);
+          }
+        }
+      }
     }
+    tile += wave_stride;
+    if (tile < n_tiles) load_tile(tile);  // lands during the epilogue
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; i++) {
@@ -330,31 +447,48 @@ __device__ __forceinline__ void rope_pair_f16(float x0, float x1, float c, float
 // float16 values widened to float32; dims >= 448 take the partial rope at float16 op rounding.
 __global__ __launch_bounds__(64) void kv_row_kernel(const uint16_t* __restrict__ kv, const float* __restrict__ inv_freq,
                                                     const int32_t* __restrict__ params, uint16_t* __restrict__ row_out) {
-  int lane32 = threadIdx.x & 31;
-  if (threadIdx.x >= 32) return;  // the shuffles below stay inside lanes 0..31 (xor 1, 2)
+  // The upper half-wave works out the 32 cosine / sine pairs, one frequency per lane, while the lower
+  // half-wave loads the row; the four rope lanes then pick their eight pairs up from LDS. (One lane
+  // doing its eight double-precision cosine / sine pairs in a row was most of this kernel's time.)
+  __shared__ float cs[32], sn[32];
+  const int lane32 = threadIdx.x & 31;
+  if (threadIdx.x >= 32) {
+    const float theta = (float)params[0] * inv_freq[lane32];
+    cs[lane32] = h_round((float)cos((double)theta));
+    sn[lane32] = h_round((float)sin((double)theta));
+  }
   float xv[16];
+  if (threadIdx.x < 32) {
+    const u32x4_t* src = reinterpret_cast<const u32x4_t*>(kv + 16 * lane32);
+    const u32x4_t w0 = src[0], w1 = src[1];
+    const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
 #pragma unroll
-  for (int j = 0; j < 16; j++) xv[j] = f16_bits_to_f32(kv[16 * lane32 + j]);
+    for (int j = 0; j < 8; j++) {
+      xv[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xFFFFu));
+      xv[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x >= 32) return;  // the shuffles below stay inside lanes 0..31 (xor 1, 2)
   float amax = block64_amax(xv);
+  float ov[16];
   if (lane32 < 28) {
     float scale = pow2_group_scale(mx_floor_max(amax, kFp8AmaxFloor), 448.0f);
 #pragma unroll
-    for (int j = 0; j < 16; j++) row_out[16 * lane32 + j] = f32_to_f16_bits(fp8_roundtrip(xv[j], scale));
+    for (int j = 0; j < 16; j++) ov[j] = fp8_roundtrip(xv[j], scale);
   } else {
-    int pos = params[0];
 #pragma unroll
     for (int j = 0; j < 8; j++) {
-      int d0 = 16 * lane32 + 2 * j;
-      int p = (d0 - 448) / 2;
-      float theta = (float)pos * inv_freq[p];
-      float c = h_round((float)cos((double)theta));
-      float s = h_round((float)sin((double)theta));
-      float r0, r1;
-      rope_pair_f16(xv[2 * j], xv[2 * j + 1], c, s, &r0, &r1);
-      row_out[d0] = f32_to_f16_bits(r0);
-      row_out[d0 + 1] = f32_to_f16_bits(r1);
+      const int p = (16 * lane32 + 2 * j - 448) / 2;
+      rope_pair_f16(xv[2 * j], xv[2 * j + 1], cs[p], sn[p], &ov[2 * j], &ov[2 * j + 1]);
     }
   }
+  uint32_t o[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) o[j] = (uint32_t)f32_to_f16_bits(ov[2 * j]) | ((uint32_t)f32_to_f16_bits(ov[2 * j + 1]) << 16);
+  u32x4_t* dst = reinterpret_cast<u32x4_t*>(row_out + 16 * lane32);
+  dst[0] = u32x4_t{o[0], o[1], o[2], o[3]};
+  dst[1] = u32x4_t{o[4], o[5], o[6], o[7]};
 }
 
 }  // namespace
@@ -388,9 +522,9 @@ extern "C" int mspr_indexer_q_qat_live(const float* q, int64_t n_rows, float* ou
 int mspr_launch_scores_f32(const void* q, int q_dtype, int n_heads, const float* pooled, int64_t n_rows,
                            const float* weights, float scale, float* scores, bool stage_half, hipStream_t st) {
   int64_t n_tiles = (n_rows + 31) / 32;
-  int64_t blocks = (n_tiles + 3) / 4;
+  int64_t blocks = (n_tiles + kScoreWaves - 1) / kScoreWaves;
   if (blocks > 2048) blocks = 2048;
-  dim3 grid((unsigned)blocks), block(256);
+  dim3 grid((unsigned)blocks), block(kScoreThreads);
   MsprProfScope prof(MSPR_K_SCORES_F32, st);
 #define MSPR_SCORES_LAUNCH(DT)                                                                          \
   do {                                                                                                  \

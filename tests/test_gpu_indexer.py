@@ -128,6 +128,29 @@ def test_fused_qat_indexer_scores_low_precision_and_few_heads():
     np.testing.assert_allclose(got, ds4.fused_qat_indexer_scores(q, pooled, w, 128 ** -0.5), rtol=1e-5, atol=1e-5)
 
 
+def test_fused_qat_indexer_scores_on_pool_rows_that_are_not_bf16_numbers():
+    # the kernel multiplies on the bf16 matrix cores; pool values with more than 8 significant bits take
+    # its exact three-piece form, tile by tile (here: mixed tiles, only rows 32..63 and the ragged tail carry
+    # arbitrary float32 values)
+    rng = np.random.default_rng(77)
+    q, pooled, w = _score_inputs(131, rng)
+    pooled = pooled.copy()
+    pooled[0, 32:64] = rng.standard_normal((32, 128), dtype=np.float32)
+    pooled[0, 128:] = rng.standard_normal((3, 128), dtype=np.float32) * 1e-3
+    got = isk.fused_qat_indexer_scores(to_dev(q), to_dev(pooled), to_dev(w), 128 ** -0.5).cpu().numpy()
+    want = ds4.fused_qat_indexer_scores(q, pooled, w, 128 ** -0.5)
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5)
+    # integer pool values up to 2^20 and integer-valued lattice queries: every product and partial sum is an
+    # exact float32 integer, so any lost piece would show
+    qi = np.zeros((1, 4, 1, 128), dtype=np.float32)
+    qi[0, :, 0, 0] = 1.0  # qat(e0) = H e0 / sqrt(128) per element: a constant row, checked through the oracle
+    big = rng.integers(-(1 << 20), 1 << 20, (1, 70, 128)).astype(np.float32)
+    wi = np.ones((1, 1, 4), dtype=np.float32)
+    got = isk.fused_qat_indexer_scores(to_dev(qi), to_dev(big), to_dev(wi), 1.0).cpu().numpy()
+    want = ds4.fused_qat_indexer_scores(qi, big, wi, 1.0)
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=0)
+
+
 def test_fused_scores_known_answer_ones():
     # qat(ones) = [12, 0, ...]: score = 144 / sqrt(128) per unit weight
     q = torch.ones((1, 2, 1, 128), device=dev())
