@@ -8,8 +8,8 @@
 // Each K row is read from HBM once and staged row-major in LDS (ring of three tiles, filled by
 // asynchronous global->LDS copies). The eight waves are (head group hg of 32 heads) x (quarter dh):
 // for S^T = K.Q^T a wave contracts its quarter of the row width and the four quarters are summed
-// through LDS; for O^T = V^T.P^T it owns 128 of the 512 output columns. Two waves share a SIMD: one
-// wave alone can issue a 32x32x16 MFMA only every other slot of the matrix pipe. V^T operands come
+// through LDS; for O^T = V^T.P^T it owns 128 of the 512 output columns. Two waves share a SIMD and
+// fill each other's waits (a wave has no matrix work while it stages or exchanges). V^T operands come
 // out of the same row-major tile through the LDS transpose read, so no second copy of the tile
 // exists. Partial (m, l, O) per slot range are merged by a second kernel (log-sum-exp), which also
 // applies the sink, the normalisation, the output cast and the optional inverse rope.
@@ -518,8 +518,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 
     MSPR_STAMP(5 + 6 * t);
     // S^T partial over this wave's half of the row width
-    // (two accumulators, even and odd k-steps: a wave is alone on its SIMD, so a single chain of
-    // dependent MFMAs would run at the instruction's latency instead of its issue rate)
+    // (two accumulators, even and odd k-steps: a single chain of dependent MFMAs runs about a tenth
+    // below the issue rate of independent ones)
     f32x16_t sacc = {0};
     {
       f32x16_t sodd = {0};
