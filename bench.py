@@ -125,8 +125,11 @@ def cpu_config1():
             "workload": "dense GQA decode, 8q/1kv heads, D=128, 4096 fp16 keys (BASELINE config 1), NumPy float64"}
 
 
-def bench_prefill(dev, gen, reps=5):
-    """BASELINE config 2: 4096-token bf16 chunk over a 32768-token prefix, 16 q / 2 KV heads, D=256."""
+def bench_prefill(dev, gen, reps=10, warmup=20):
+    """BASELINE config 2: 4096-token bf16 chunk over a 32768-token prefix, 16 q / 2 KV heads, D=256.
+
+    The launches run back to back; the first ones after lighter work are about a tenth slower than the
+    sustained rate, hence the warm-up."""
     from moespresso_amd import _lib
     from moespresso_amd.runtime.qwen import kquant
 
@@ -134,7 +137,7 @@ def bench_prefill(dev, gen, reps=5):
     q = (0.5 * torch.randn((1, 16, L, 256), device=dev, generator=gen)).to(torch.bfloat16)
     k = (0.5 * torch.randn((1, 2, past + L, 256), device=dev, generator=gen)).to(torch.bfloat16)
     v = (0.5 * torch.randn((1, 2, past + L, 256), device=dev, generator=gen)).to(torch.bfloat16)
-    for _ in range(2):
+    for _ in range(warmup):
         kquant.flash_prefill(q, k, v, 256 ** -0.5, past_len=past)
     torch.cuda.synchronize()
     _lib.profile_enable("flash_prefill")
