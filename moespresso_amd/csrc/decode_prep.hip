@@ -1,11 +1,12 @@
-// Host entry of the fused ratio-4 decode prep: three launches on one stream (score row with the
-// query QAT staged as float16, prepared KV row, radix top-k). The reference runs the same phases
-// inside a single 1024-thread workgroup; here the score row is spread over the whole device.
+// Host entry of the fused ratio-4 decode prep: two launches on one stream (score row with the query
+// QAT staged as float16, with the prepared KV row as one more workgroup of the same launch; radix
+// top-k). The reference runs the same phases inside a single 1024-thread workgroup; here the score
+// row is spread over the whole device.
 #include "common.h"
 
 int mspr_launch_scores_f32(const void* q, int q_dtype, int n_heads, const float* pooled, int64_t n_rows,
-                           const float* weights, float scale, float* scores, bool stage_half, hipStream_t st);
-int mspr_launch_kv_row(const void* kv_row, const float* inv_freq, const int32_t* params, void* row_out, hipStream_t st);
+                           const float* weights, float scale, float* scores, bool stage_half, const void* kv_row,
+                           const float* inv_freq, const int32_t* params, void* row_out, hipStream_t st);
 int mspr_launch_topk(const float* scores, int64_t score_stride, int batch, int64_t n_rows, int topk, int32_t* sel,
                      hipStream_t st);
 
@@ -23,9 +24,8 @@ extern "C" int mspr_fused_decode_prep(const void* q_idx, int q_dtype, int n_head
                    mspr_aligned(row_out, 16),
                "fused_decode_prep: q_idx, pooled_qat, kv_row and row_out must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  int rc = mspr_launch_scores_f32(q_idx, q_dtype, n_heads, pooled_qat, n_rows, weights, scale, scores, true, st);
-  if (rc != MSPR_OK) return rc;
-  rc = mspr_launch_kv_row(kv_row, inv_freq, params, row_out, st);
+  int rc = mspr_launch_scores_f32(q_idx, q_dtype, n_heads, pooled_qat, n_rows, weights, scale, scores, true, kv_row,
+                                  inv_freq, params, row_out, st);
   if (rc != MSPR_OK) return rc;
   return mspr_launch_topk(scores, n_rows, 1, n_rows, topk, sel, st);
 }

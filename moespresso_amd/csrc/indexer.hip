@@ -155,6 +155,161 @@ __global__ __launch_bounds__(256) void qat_rows_kernel(const void* __restrict__ 
   if (row < n_rows) reinterpret_cast<f32x4_t*>(out + row * 128)[lane32] = y;
 }
 
+// ------------------------------------------------------------------ score tail
+template <int WDT>
+__global__ __launch_bounds__(256) void score_tail_kernel(const float* __restrict__ s, int n_heads,
+                                                         int64_t capacity, const void* __restrict__ wraw,
+                                                         const int32_t* __restrict__ params, float scale,
+                                                         float head_norm, float* __restrict__ neg) {
+  int lane32 = threadIdx.x & 31;
+  int64_t col = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+  int64_t c = col < capacity ? col : capacity - 1;
+  int32_t pv = params[1];
+  int64_t valid = pv < 0 ? 0 : (pv < capacity ? pv : capacity);
+  float partial = 0.0f;
+  for (int h = lane32; h < n_heads; h += 32) {
+    float w = mul_rn(load_as_f32<WDT>(wraw, h), head_norm);
+    float t = s[(int64_t)h * capacity + c];
+    t = isnan(t) ? t : (t > 0.0f ? t : 0.0f);
+    t = mul_rn(t, scale);
+    t = mul_rn(t, w);
+    partial = add_rn(partial, t);
+  }
+#pragma unroll
+  for (int off = 16; off >= 1; off >>= 1) partial = add_rn(partial, __shfl_xor(partial, off, MSPR_WAVE));
+  if (lane32 == 0 && col < capacity) neg[col] = col < valid ? -partial : __builtin_inff();
+}
+
+// ------------------------------------------------------------------ E4M3FN round trip
+// Nearest non-negative E4M3FN value of a in [0, 448]; exact ties go to the lower value. Equal to
+// a first-wins scan of the ascending 127-entry table: both neighbours' distances are exact in
+// float32, so only they can win.
+__device__ __forceinline__ float e4m3_nearest_lower_ties(float a) {
+  if (isnan(a)) return 0.0f;  // a scan that compares against NaN keeps entry 0
+  float lo, step;
+  if (a < 0.015625f) {
+    step = 0.001953125f;
+    lo = floorf(a * 512.0f) * 0.001953125f;
+  } else {
+    uint32_t u = __float_as_uint(a);
+    lo = __uint_as_float(u & 0xFFF00000u);
+    step = __uint_as_float((u & 0x7F800000u) - (3u << 23));
+  }
+  if (lo >= 448.0f) return 448.0f;
+  float hi = lo + step;
+  return (hi - a) < (a - lo) ? hi : lo;
+}
+
+__device__ __forceinline__ float fp8_roundtrip(float x, float scale) {
+  float n = x / scale;
+  n = (isnan(n) || n > -448.0f) ? n : -448.0f;
+  n = (isnan(n) || n < 448.0f) ? n : 448.0f;
+  float qv = e4m3_nearest_lower_ties(fabsf(n));
+  float sign = n < 0.0f ? -1.0f : (n > 0.0f ? 1.0f : 0.0f);
+  return mul_rn(mul_rn(sign, qv), scale);
+}
+
+// amax over a 64-element block = 4 lanes x 16 values.
+__device__ __forceinline__ float block64_amax(const float (&xv)[16]) {
+  float amax = 0.0f;
+#pragma unroll
+  for (int j = 0; j < 16; j++) amax = fmaxf(amax, fabsf(xv[j]));
+  amax = fmaxf(amax, __shfl_xor(amax, 1, MSPR_WAVE));
+  amax = fmaxf(amax, __shfl_xor(amax, 2, MSPR_WAVE));
+  return amax;
+}
+
+__global__ __launch_bounds__(256) void fp8_rows_kernel(const float* __restrict__ x, int64_t n_rows,
+                                                       float* __restrict__ out) {
+  int lane32 = threadIdx.x & 31;
+  int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+  int64_t src = row < n_rows ? row : n_rows - 1;
+  const f32x4_t* xp = reinterpret_cast<const f32x4_t*>(x + src * 512 + 16 * lane32);
+  float xv[16];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    f32x4_t t = xp[j];
+    xv[4 * j] = t.x;
+    xv[4 * j + 1] = t.y;
+    xv[4 * j + 2] = t.z;
+    xv[4 * j + 3] = t.w;
+  }
+  float amax = block64_amax(xv);
+  float ov[16];
+  if (lane32 < 28) {
+    float scale = pow2_group_scale(mx_floor_max(amax, kFp8AmaxFloor), 448.0f);
+#pragma unroll
+    for (int j = 0; j < 16; j++) ov[j] = fp8_roundtrip(xv[j], scale);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 16; j++) ov[j] = xv[j];
+  }
+  if (row < n_rows) {
+    f32x4_t* op = reinterpret_cast<f32x4_t*>(out + row * 512 + 16 * lane32);
+#pragma unroll
+    for (int j = 0; j < 4; j++) op[j] = f32x4_t{ov[4 * j], ov[4 * j + 1], ov[4 * j + 2], ov[4 * j + 3]};
+  }
+}
+
+// ------------------------------------------------------------------ prepared KV row
+__device__ __forceinline__ float h_round(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
+
+// One (even, odd) pair rotated with every product and sum rounded to float16.
+__device__ __forceinline__ void rope_pair_f16(float x0, float x1, float c, float s, float* o0, float* o1) {
+  float m0 = h_round(x0 * c), m1 = h_round(x1 * s), m2 = h_round(x0 * s), m3 = h_round(x1 * c);
+  *o0 = h_round(m0 - m1);
+  *o1 = h_round(m2 + m3);
+}
+
+// Prepared KV row of the decode island, one job for the first wave of a workgroup (every thread of the
+// workgroup calls this and reaches its one barrier). Lane l of the lower half-wave holds dims
+// [16l, 16l+16): dims < 448 take the E4M3FN round trip of the float16 values widened to float32, dims
+// >= 448 the partial rope at float16 op rounding. The upper half-wave works out the 32 cosine / sine
+// pairs, one frequency per lane, while the lower one loads the row; the four rope lanes then pick their
+// eight pairs up from LDS (cs, sn: 32 floats each).
+__device__ __forceinline__ void kv_row_job(int tid, float* cs, float* sn, const uint16_t* __restrict__ kv,
+                                           const float* __restrict__ inv_freq, const int32_t* __restrict__ params,
+                                           uint16_t* __restrict__ row_out) {
+  const int lane32 = tid & 31;
+  if (tid >= 32 && tid < 64) {
+    const float theta = (float)params[0] * inv_freq[lane32];
+    cs[lane32] = h_round((float)cos((double)theta));
+    sn[lane32] = h_round((float)sin((double)theta));
+  }
+  float xv[16];
+  if (tid < 32) {
+    const u32x4_t* src = reinterpret_cast<const u32x4_t*>(kv + 16 * lane32);
+    const u32x4_t w0 = src[0], w1 = src[1];
+    const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      xv[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xFFFFu));
+      xv[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+    }
+  }
+  __syncthreads();
+  if (tid >= 32) return;  // the shuffles below stay inside lanes 0..31 (xor 1, 2)
+  float amax = block64_amax(xv);
+  float ov[16];
+  if (lane32 < 28) {
+    float scale = pow2_group_scale(mx_floor_max(amax, kFp8AmaxFloor), 448.0f);
+#pragma unroll
+    for (int j = 0; j < 16; j++) ov[j] = fp8_roundtrip(xv[j], scale);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int p = (16 * lane32 + 2 * j - 448) / 2;
+      rope_pair_f16(xv[2 * j], xv[2 * j + 1], cs[p], sn[p], &ov[2 * j], &ov[2 * j + 1]);
+    }
+  }
+  uint32_t o[8];
+#pragma unroll
+  for (int j = 0; j < 8; j++) o[j] = (uint32_t)f32_to_f16_bits(ov[2 * j]) | ((uint32_t)f32_to_f16_bits(ov[2 * j + 1]) << 16);
+  u32x4_t* dst = reinterpret_cast<u32x4_t*>(row_out + 16 * lane32);
+  dst[0] = u32x4_t{o[0], o[1], o[2], o[3]};
+  dst[1] = u32x4_t{o[4], o[5], o[6], o[7]};
+}
+
 // ------------------------------------------------------------------ score row, float32 pool rows
 // Block = 8 waves. The block QATs the (up to 64) query heads into LDS once (four rows per lane, while
 // the wave's first pool tile is already on its way), each wave then keeps them in registers as the
@@ -182,11 +337,22 @@ template <int DT, bool STAGE_HALF>
 __global__ __launch_bounds__(kScoreThreads) void scores_f32_kernel(const void* __restrict__ q, int n_heads,
                                                                    const float* __restrict__ pooled, int64_t n_rows,
                                                                    const float* __restrict__ weights, float scale,
-                                                                   float* __restrict__ scores) {
+                                                                   float* __restrict__ scores,
+                                                                   const uint16_t* __restrict__ kv_row,
+                                                                   const float* __restrict__ inv_freq,
+                                                                   const int32_t* __restrict__ params,
+                                                                   uint16_t* __restrict__ row_out) {
   __shared__ float qbuf[64 * kQPitch];
   __shared__ float wbuf[64];
   __shared__ float ptab[kPow2TabLen];
   const int tid = threadIdx.x;
+  // With a KV row to prepare (the fused decode prep), the launch carries one more workgroup, the last one,
+  // whose first wave does that small job next to the score workgroups instead of in a launch of its own.
+  const int score_blocks = (int)gridDim.x - (kv_row ? 1 : 0);
+  if ((int)blockIdx.x == score_blocks) {
+    kv_row_job(tid, qbuf, qbuf + 32, kv_row, inv_freq, params, row_out);
+    return;
+  }
   const int lane = tid & 63;
   const int lane32 = tid & 31;
   const int wave = tid >> 6;
@@ -195,7 +361,7 @@ __global__ __launch_bounds__(kScoreThreads) void scores_f32_kernel(const void* _
   const int g = lane >> 5;
 
   const int64_t n_tiles = (n_rows + 31) / 32;
-  const int64_t wave_stride = (int64_t)gridDim.x * kScoreWaves;
+  const int64_t wave_stride = (int64_t)score_blocks * kScoreWaves;
   int64_t tile = (int64_t)blockIdx.x * kScoreWaves + wave;
 
   // The eight waves QAT the 64 query rows, one row per half-wave and four rows per lane; the rows of a
@@ -337,160 +503,6 @@ __global__ __launch_bounds__(kScoreThreads) void scores_f32_kernel(const void* _
   }
 }
 
-// ------------------------------------------------------------------ score tail
-template <int WDT>
-__global__ __launch_bounds__(256) void score_tail_kernel(const float* __restrict__ s, int n_heads,
-                                                         int64_t capacity, const void* __restrict__ wraw,
-                                                         const int32_t* __restrict__ params, float scale,
-                                                         float head_norm, float* __restrict__ neg) {
-  int lane32 = threadIdx.x & 31;
-  int64_t col = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
-  int64_t c = col < capacity ? col : capacity - 1;
-  int32_t pv = params[1];
-  int64_t valid = pv < 0 ? 0 : (pv < capacity ? pv : capacity);
-  float partial = 0.0f;
-  for (int h = lane32; h < n_heads; h += 32) {
-    float w = mul_rn(load_as_f32<WDT>(wraw, h), head_norm);
-    float t = s[(int64_t)h * capacity + c];
-    t = isnan(t) ? t : (t > 0.0f ? t : 0.0f);
-    t = mul_rn(t, scale);
-    t = mul_rn(t, w);
-    partial = add_rn(partial, t);
-  }
-#pragma unroll
-  for (int off = 16; off >= 1; off >>= 1) partial = add_rn(partial, __shfl_xor(partial, off, MSPR_WAVE));
-  if (lane32 == 0 && col < capacity) neg[col] = col < valid ? -partial : __builtin_inff();
-}
-
-// ------------------------------------------------------------------ E4M3FN round trip
-// Nearest non-negative E4M3FN value of a in [0, 448]; exact ties go to the lower value. Equal to
-// a first-wins scan of the ascending 127-entry table: both neighbours' distances are exact in
-// float32, so only they can win.
-__device__ __forceinline__ float e4m3_nearest_lower_ties(float a) {
-  if (isnan(a)) return 0.0f;  // a scan that compares against NaN keeps entry 0
-  float lo, step;
-  if (a < 0.015625f) {
-    step = 0.001953125f;
-    lo = floorf(a * 512.0f) * 0.001953125f;
-  } else {
-    uint32_t u = __float_as_uint(a);
-    lo = __uint_as_float(u & 0xFFF00000u);
-    step = __uint_as_float((u & 0x7F800000u) - (3u << 23));
-  }
-  if (lo >= 448.0f) return 448.0f;
-  float hi = lo + step;
-  return (hi - a) < (a - lo) ? hi : lo;
-}
-
-__device__ __forceinline__ float fp8_roundtrip(float x, float scale) {
-  float n = x / scale;
-  n = (isnan(n) || n > -448.0f) ? n : -448.0f;
-  n = (isnan(n) || n < 448.0f) ? n : 448.0f;
-  float qv = e4m3_nearest_lower_ties(fabsf(n));
-  float sign = n < 0.0f ? -1.0f : (n > 0.0f ? 1.0f : 0.0f);
-  return mul_rn(mul_rn(sign, qv), scale);
-}
-
-// amax over a 64-element block = 4 lanes x 16 values.
-__device__ __forceinline__ float block64_amax(const float (&xv)[16]) {
-  float amax = 0.0f;
-#pragma unroll
-  for (int j = 0; j < 16; j++) amax = fmaxf(amax, fabsf(xv[j]));
-  amax = fmaxf(amax, __shfl_xor(amax, 1, MSPR_WAVE));
-  amax = fmaxf(amax, __shfl_xor(amax, 2, MSPR_WAVE));
-  return amax;
-}
-
-__global__ __launch_bounds__(256) void fp8_rows_kernel(const float* __restrict__ x, int64_t n_rows,
-                                                       float* __restrict__ out) {
-  int lane32 = threadIdx.x & 31;
-  int64_t row = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
-  int64_t src = row < n_rows ? row : n_rows - 1;
-  const f32x4_t* xp = reinterpret_cast<const f32x4_t*>(x + src * 512 + 16 * lane32);
-  float xv[16];
-#pragma unroll
-  for (int j = 0; j < 4; j++) {
-    f32x4_t t = xp[j];
-    xv[4 * j] = t.x;
-    xv[4 * j + 1] = t.y;
-    xv[4 * j + 2] = t.z;
-    xv[4 * j + 3] = t.w;
-  }
-  float amax = block64_amax(xv);
-  float ov[16];
-  if (lane32 < 28) {
-    float scale = pow2_group_scale(mx_floor_max(amax, kFp8AmaxFloor), 448.0f);
-#pragma unroll
-    for (int j = 0; j < 16; j++) ov[j] = fp8_roundtrip(xv[j], scale);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 16; j++) ov[j] = xv[j];
-  }
-  if (row < n_rows) {
-    f32x4_t* op = reinterpret_cast<f32x4_t*>(out + row * 512 + 16 * lane32);
-#pragma unroll
-    for (int j = 0; j < 4; j++) op[j] = f32x4_t{ov[4 * j], ov[4 * j + 1], ov[4 * j + 2], ov[4 * j + 3]};
-  }
-}
-
-// ------------------------------------------------------------------ prepared KV row
-__device__ __forceinline__ float h_round(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
-
-// One (even, odd) pair rotated with every product and sum rounded to float16.
-__device__ __forceinline__ void rope_pair_f16(float x0, float x1, float c, float s, float* o0, float* o1) {
-  float m0 = h_round(x0 * c), m1 = h_round(x1 * s), m2 = h_round(x0 * s), m3 = h_round(x1 * c);
-  *o0 = h_round(m0 - m1);
-  *o1 = h_round(m2 + m3);
-}
-
-// One half-wave: lane l holds dims [16l, 16l+16). Dims < 448 take the E4M3FN round trip of the
-// float16 values widened to float32; dims >= 448 take the partial rope at float16 op rounding.
-__global__ __launch_bounds__(64) void kv_row_kernel(const uint16_t* __restrict__ kv, const float* __restrict__ inv_freq,
-                                                    const int32_t* __restrict__ params, uint16_t* __restrict__ row_out) {
-  // The upper half-wave works out the 32 cosine / sine pairs, one frequency per lane, while the lower
-  // half-wave loads the row; the four rope lanes then pick their eight pairs up from LDS. (One lane
-  // doing its eight double-precision cosine / sine pairs in a row was most of this kernel's time.)
-  __shared__ float cs[32], sn[32];
-  const int lane32 = threadIdx.x & 31;
-  if (threadIdx.x >= 32) {
-    const float theta = (float)params[0] * inv_freq[lane32];
-    cs[lane32] = h_round((float)cos((double)theta));
-    sn[lane32] = h_round((float)sin((double)theta));
-  }
-  float xv[16];
-  if (threadIdx.x < 32) {
-    const u32x4_t* src = reinterpret_cast<const u32x4_t*>(kv + 16 * lane32);
-    const u32x4_t w0 = src[0], w1 = src[1];
-    const uint32_t w[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      xv[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xFFFFu));
-      xv[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
-    }
-  }
-  __syncthreads();
-  if (threadIdx.x >= 32) return;  // the shuffles below stay inside lanes 0..31 (xor 1, 2)
-  float amax = block64_amax(xv);
-  float ov[16];
-  if (lane32 < 28) {
-    float scale = pow2_group_scale(mx_floor_max(amax, kFp8AmaxFloor), 448.0f);
-#pragma unroll
-    for (int j = 0; j < 16; j++) ov[j] = fp8_roundtrip(xv[j], scale);
-  } else {
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const int p = (16 * lane32 + 2 * j - 448) / 2;
-      rope_pair_f16(xv[2 * j], xv[2 * j + 1], cs[p], sn[p], &ov[2 * j], &ov[2 * j + 1]);
-    }
-  }
-  uint32_t o[8];
-#pragma unroll
-  for (int j = 0; j < 8; j++) o[j] = (uint32_t)f32_to_f16_bits(ov[2 * j]) | ((uint32_t)f32_to_f16_bits(ov[2 * j + 1]) << 16);
-  u32x4_t* dst = reinterpret_cast<u32x4_t*>(row_out + 16 * lane32);
-  dst[0] = u32x4_t{o[0], o[1], o[2], o[3]};
-  dst[1] = u32x4_t{o[4], o[5], o[6], o[7]};
-}
-
 }  // namespace
 
 // ====================================================================== C-ABI
@@ -519,19 +531,25 @@ extern "C" int mspr_indexer_q_qat_live(const float* q, int64_t n_rows, float* ou
   return MSPR_OK;
 }
 
+// kv_row (with inv_freq, params, row_out) may be null: no prepared KV row in this launch
 int mspr_launch_scores_f32(const void* q, int q_dtype, int n_heads, const float* pooled, int64_t n_rows,
-                           const float* weights, float scale, float* scores, bool stage_half, hipStream_t st) {
+                           const float* weights, float scale, float* scores, bool stage_half, const void* kv_row,
+                           const float* inv_freq, const int32_t* params, void* row_out, hipStream_t st) {
   int64_t n_tiles = (n_rows + 31) / 32;
   int64_t blocks = (n_tiles + kScoreWaves - 1) / kScoreWaves;
   if (blocks > 2048) blocks = 2048;
-  dim3 grid((unsigned)blocks), block(kScoreThreads);
+  dim3 grid((unsigned)(blocks + (kv_row ? 1 : 0))), block(kScoreThreads);
+  const uint16_t* kvp = reinterpret_cast<const uint16_t*>(kv_row);
+  uint16_t* rop = reinterpret_cast<uint16_t*>(row_out);
   MsprProfScope prof(MSPR_K_SCORES_F32, st);
 #define MSPR_SCORES_LAUNCH(DT)                                                                          \
   do {                                                                                                  \
     if (stage_half)                                                                                     \
-      scores_f32_kernel<DT, true><<<grid, block, 0, st>>>(q, n_heads, pooled, n_rows, weights, scale, scores);  \
+      scores_f32_kernel<DT, true><<<grid, block, 0, st>>>(q, n_heads, pooled, n_rows, weights, scale, scores, kvp, \
+                                                          inv_freq, params, rop);                        \
     else                                                                                                \
-      scores_f32_kernel<DT, false><<<grid, block, 0, st>>>(q, n_heads, pooled, n_rows, weights, scale, scores); \
+      scores_f32_kernel<DT, false><<<grid, block, 0, st>>>(q, n_heads, pooled, n_rows, weights, scale, scores, kvp, \
+                                                           inv_freq, params, rop);                        \
   } while (0)
   if (q_dtype == MSPR_F32) MSPR_SCORES_LAUNCH(MSPR_F32);
   else if (q_dtype == MSPR_F16) MSPR_SCORES_LAUNCH(MSPR_F16);
@@ -549,8 +567,8 @@ extern "C" int mspr_fused_qat_indexer_scores(const void* q, int q_dtype, int n_h
   MSPR_REQUIRE(n_rows > 0, "fused_qat_indexer_scores: pooled_qat must contain at least one row");
   MSPR_REQUIRE(q_dtype >= MSPR_F32 && q_dtype <= MSPR_BF16, "fused_qat_indexer_scores: q must be f32, f16 or bf16");
   MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(pooled_qat, 16), "fused_qat_indexer_scores: q and pooled_qat must be 16-byte aligned");
-  return mspr_launch_scores_f32(q, q_dtype, n_heads, pooled_qat, n_rows, weights, scale, scores, false,
-                                (hipStream_t)stream);
+  return mspr_launch_scores_f32(q, q_dtype, n_heads, pooled_qat, n_rows, weights, scale, scores, false, nullptr,
+                                nullptr, nullptr, nullptr, (hipStream_t)stream);
 }
 
 extern "C" int mspr_indexer_score_tail(const float* scores, int n_heads, int64_t capacity, const void* weights_raw,
@@ -579,9 +597,3 @@ extern "C" int mspr_fp8_kv_prefix_rows(const float* x, int64_t n_rows, float* ou
   return MSPR_OK;
 }
 
-int mspr_launch_kv_row(const void* kv_row, const float* inv_freq, const int32_t* params, void* row_out, hipStream_t st) {
-  kv_row_kernel<<<1, 64, 0, st>>>(reinterpret_cast<const uint16_t*>(kv_row), inv_freq, params,
-                                  reinterpret_cast<uint16_t*>(row_out));
-  MSPR_CHECK_LAUNCH("prepared kv row");
-  return MSPR_OK;
-}
