@@ -114,6 +114,32 @@ __device__ __forceinline__ float lane_xor(float v) {
   return __int_as_float(x);
 }
 
+// max / sum of a value over the two half-waves (lane l with lane l ^ 32), the same result in both lanes.
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second: with
+// two copies of the value, each lane ends up holding its own and its partner's value in the two registers.
+// A vector-ALU exchange, so no LDS round trip as with the general lane permute. (The waits around it are
+// the distance the instruction needs from vector writes of its operands and to reads of its results.)
+__device__ __forceinline__ void half_wave_exchange(float& a, float& b) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float half_wave_max(float v) {
+  float w = v;
+  half_wave_exchange(v, w);
+  return fmaxf(v, w);
+}
+// the same over lanes l and l ^ 16 (v_permlane16_swap: odd rows of 16 lanes of the first operand with the
+// even rows of the second)
+__device__ __forceinline__ float row_pair_max(float v) {
+  float w = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(v), "+v"(w));
+  return fmaxf(v, w);
+}
+__device__ __forceinline__ float half_wave_sum(float v) {
+  float w = v;
+  half_wave_exchange(v, w);
+  return v + w;
+}
+
 // Monotone float32 -> uint32 map: negatives inverted, positives offset. Orders -0.0 below +0.0
 // and +NaN above +inf.
 __device__ __forceinline__ uint32_t score_key(float s) {

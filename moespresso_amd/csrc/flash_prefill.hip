@@ -275,7 +275,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
         tmax = fmaxf(tmax, sacc[i]);
       }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, MSPR_WAVE)) * a.scale_log2;
+    tmax = half_wave_max(tmax) * a.scale_log2;
     constexpr float kGrow = KDT == MSPR_BF16 ? 64.0f : 8.0f;
     const bool grow = tmax > m_run + kGrow;
     if (__any(grow)) {

@@ -292,8 +292,7 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
         sacc[u][i] = valid ? sacc[u][i] : -__builtin_inff();
         tmax = fmaxf(tmax, sacc[u][i]);
       }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, MSPR_WAVE));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, MSPR_WAVE));
+    tmax = half_wave_max(row_pair_max(tmax));
     const bool grow = tmax > m_run + 8.0f;
     if (__any(grow)) {
       const float m_new = grow ? tmax : m_run;

@@ -591,7 +591,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         tmax = fmaxf(tmax, sacc[i]);
       }
     }
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, MSPR_WAVE));
+    tmax = half_wave_max(tmax);
     // bf16 weights keep float32's exponent range, float16 weights must stay below 2^15
     constexpr float kGrow = KDT == MSPR_BF16 ? 64.0f : 8.0f;
     const bool grow = tmax > m_run + kGrow;
