@@ -116,6 +116,17 @@ __device__ __forceinline__ void async_load_16(uint64_t base, uint32_t offset, ui
                : "memory", "m0");
 }
 
+// the same with 4 bytes per lane: lane i's dword lands at lds_base + 4 i
+__device__ __forceinline__ void async_load_4(uint64_t base, uint32_t offset, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %1, %0" ::"s"(base), "v"(offset), "s"(lds_base)
+               : "memory", "m0");
+}
+
+// LDS byte address of a pointer into the kernel's dynamic LDS
+__device__ __forceinline__ uint32_t lds_addr(const unsigned char* p) {
+  return (uint32_t)(uintptr_t)MSPR_LDS_PTR(const unsigned char, p);
+}
+
 // swizzle of the 16-byte pieces of a tile row: piece p of row r sits at slot (p & 16) | ((p ^ f(r)) & 15)
 __device__ __forceinline__ int swz(int r) { return ((r & 7) << 1) | ((r >> 3) & 1); }
 
@@ -123,7 +134,7 @@ __device__ __forceinline__ int swz(int r) { return ((r & 7) << 1) | ((r >> 3) & 
 // Q8 = true (KDT float16): float32 q / out, quantised prefix + float16 tail rows (see PrefillArgs).
 template <int KDT, bool Q8, int SDT>
 __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs a) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  extern __shared__ __attribute__((aligned(256))) unsigned char lds[];  // tile bases: zero low bits under the address XORs
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -232,7 +243,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
     v_off[h] = kTileBytes + r * kRowBytes + 16 * ((tr_piece ^ swz(r)) & 15) + 8 * (tr_s & 1);
   }
   const int my_last_key = past + q0 + 31;  // last key any query of this wave may see
-  const int qpos = past + q0 + n;
+  const int qpos_g = past + q0 + n - 4 * g;  // the lane's query position minus its key offset inside a tile
 
   // stage 1 of a tile: S^T = K . Q^T on the matrix cores
   auto qk_tile = [&](const unsigned char* st, f32x16_t& sacc) {
@@ -242,11 +253,17 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
       // all sixteen K operand reads are written out up front; the scheduling directives below make
       // the compiler keep kAhead of them in flight in front of the dependent MFMA chain instead of
       // waiting for each read right before its MFMA
-      constexpr int kAhead = 4;
+#ifndef MSPR_FP_AHEAD_K
+#define MSPR_FP_AHEAD_K 4
+#endif
+      constexpr int kAhead = MSPR_FP_AHEAD_K;
+      // (the k-step enters the address by XOR on top of the tile base: formed per tile, the eight variants
+      // are not carried in registers across the loop)
+      const uint32_t kb = lds_addr(st) + (uint32_t)k_off;
       u32x4_t af[16];
 #pragma unroll
       for (int s2 = 0; s2 < 16; s2++)
-        af[s2] = *reinterpret_cast<const u32x4_t*>(st + ((k_off ^ ((s2 & 7) << 5)) + (s2 >> 3) * 256));
+        af[s2] = *MSPR_LDS_PTR(const u32x4_t, (uintptr_t)((kb ^ (uint32_t)((s2 & 7) << 5)) + (uint32_t)((s2 >> 3) * 256)));
 #pragma unroll
       for (int s2 = 0; s2 < 16; s2++) sacc = mfma32<KDT>(af[s2], qf[s2], sacc);
       __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);  // DS reads
@@ -270,7 +287,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
     } else {
 #pragma unroll
       for (int i = 0; i < 16; i++) {
-        const bool valid = key0 + 8 * (i / 4) + 4 * g + (i % 4) <= qpos;
+        const bool valid = key0 + 8 * (i / 4) + (i % 4) <= qpos_g;
         sacc[i] = valid ? sacc[i] : -__builtin_inff();
         tmax = fmaxf(tmax, sacc[i]);
       }
@@ -302,16 +319,20 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
 
     // O^T += V^T . P^T; the transpose reads run kAheadV MFMAs in front of their use
     {
-      constexpr int kAheadV = 4;
+#ifndef MSPR_FP_AHEAD_V
+#define MSPR_FP_AHEAD_V 4
+#endif
+      constexpr int kAheadV = MSPR_FP_AHEAD_V;
+      const uint32_t vb0 = lds_addr(st) + (uint32_t)v_off[0], vb1 = lds_addr(st) + (uint32_t)v_off[1];
       u32x4_t vf[16];
 #pragma unroll
       for (int mt = 0; mt < 8; mt++) {
 #pragma unroll
         for (int ks = 0; ks < 2; ks++) {
-          const unsigned char* lo_p = st + ((v_off[0] ^ ((mt & 3) << 6)) + (mt >> 2) * 256 + ks * 16 * kRowBytes);
-          const unsigned char* hi_p = st + ((v_off[1] ^ ((mt & 3) << 6)) + (mt >> 2) * 256 + ks * 16 * kRowBytes);
-          s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, lo_p));
-          s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, hi_p));
+          const uint32_t lo_a = (vb0 ^ (uint32_t)((mt & 3) << 6)) + (uint32_t)((mt >> 2) * 256 + ks * 16 * kRowBytes);
+          const uint32_t hi_a = (vb1 ^ (uint32_t)((mt & 3) << 6)) + (uint32_t)((mt >> 2) * 256 + ks * 16 * kRowBytes);
+          s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, (uintptr_t)lo_a));
+          s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, (uintptr_t)hi_a));
           u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
           vf[2 * mt + ks] = u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y};
         }
@@ -336,42 +357,57 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   };
 
   if constexpr (Q8) {
-    // ---- quantised prefix: tile t+1 is unpacked from registers into the other LDS slot at the top of
-    //      step t while the raw bytes of tile t+2 are already on their way
+    // ---- quantised prefix. The raw bytes of a tile (8 KB of K codes, 8 KB of V codes, scales and biases)
+    //      are copied asynchronously into a three-slot ring in the upper half of the LDS, three tiles ahead;
+    //      tile t+1 is unpacked from there into the other float16 stage at the top of step t. No register
+    //      carries raw bytes across a step (twelve more live registers did not fit next to the accumulators,
+    //      and a spill of a freshly loaded value waits for the whole memory latency once per tile).
     const int p_end = n_tiles < t1 ? n_tiles : t1;  // prefix tiles of this workgroup: [t_begin, p_end)
     if (t_begin < p_end) {
-      const int s_row = tid >> 4;   // tile row staged by this thread
-      const int s_pp = tid & 15;    // its 16 elements: [16 s_pp, +16), scale group s_pp / 4
+      constexpr int kSB = SDT == MSPR_F32 ? 4 : 2;   // bytes per scale / bias
+      constexpr int kCodeBytes = kTile * kD;         // 8 KB of codes per tile, K and V each
+      constexpr int kScaleBytes = kTile * 4 * kSB;   // one tile of one scale or bias array: 256 or 512 B
+      constexpr int kRawBytes = 2 * kCodeBytes + 4 * 512;
+      constexpr int kRawBase = 2 * kStageBytes;      // the unpacked stages use the lower 64 KB
+      static_assert(kRawBase + 3 * kRawBytes <= kLdsBytes, "raw ring does not fit");
       const int64_t row0 = ((int64_t)b * a.n_kv_heads + kvh) * past;
-      const uint8_t* kc = reinterpret_cast<const uint8_t*>(a.pk_wq) + row0 * kD + 16 * s_pp;
-      const uint8_t* vc = reinterpret_cast<const uint8_t*>(a.pv_wq) + row0 * kD + 16 * s_pp;
-      constexpr int kSB = SDT == MSPR_F32 ? 4 : 2;
-      const uint8_t* ks = reinterpret_cast<const uint8_t*>(a.pk_s) + (row0 * 4 + (s_pp >> 2)) * kSB;
-      const uint8_t* kb = reinterpret_cast<const uint8_t*>(a.pk_b) + (row0 * 4 + (s_pp >> 2)) * kSB;
-      const uint8_t* vs = reinterpret_cast<const uint8_t*>(a.pv_s) + (row0 * 4 + (s_pp >> 2)) * kSB;
-      const uint8_t* vb = reinterpret_cast<const uint8_t*>(a.pv_b) + (row0 * 4 + (s_pp >> 2)) * kSB;
-      const int f = swz(s_row);
-      const int w_off0 = s_row * kRowBytes + 16 * (((2 * s_pp) & 16) | (((2 * s_pp) ^ f) & 15));
-      const int w_off1 = s_row * kRowBytes + 16 * (((2 * s_pp + 1) & 16) | (((2 * s_pp + 1) ^ f) & 15));
-      u32x4_t rk, rv;
-      uint32_t rs[4];
-      auto load_raw = [&](int t) {
-        const int64_t key = (int64_t)t * kTile + s_row;  // < past: only whole prefix tiles come through here
-        rk = *reinterpret_cast<const u32x4_t*>(kc + key * kD);
-        rv = *reinterpret_cast<const u32x4_t*>(vc + key * kD);
-        if constexpr (SDT == MSPR_F32) {
-          rs[0] = *reinterpret_cast<const uint32_t*>(ks + key * 16);
-          rs[1] = *reinterpret_cast<const uint32_t*>(kb + key * 16);
-          rs[2] = *reinterpret_cast<const uint32_t*>(vs + key * 16);
-          rs[3] = *reinterpret_cast<const uint32_t*>(vb + key * 16);
-        } else {
-          rs[0] = *reinterpret_cast<const uint16_t*>(ks + key * 8);
-          rs[1] = *reinterpret_cast<const uint16_t*>(kb + key * 8);
-          rs[2] = *reinterpret_cast<const uint16_t*>(vs + key * 8);
-          rs[3] = *reinterpret_cast<const uint16_t*>(vb + key * 8);
-        }
+      const uint8_t* kc = reinterpret_cast<const uint8_t*>(a.pk_wq) + row0 * kD;
+      const uint8_t* vc = reinterpret_cast<const uint8_t*>(a.pv_wq) + row0 * kD;
+      // scale / bias copies: wave w moves array w & 3 (K scale, K bias, V scale, V bias), 4 bytes per lane; with
+      // float32 scales waves 4-7 move the second 256 bytes, with 16-bit ones they repeat the copy of waves 0-3
+      // (every wave then issues the same number of copies and the waits below are static counts)
+      const int arr = wave & 3;
+      const uint8_t* sb_base = reinterpret_cast<const uint8_t*>(arr == 0 ? a.pk_s : arr == 1 ? a.pk_b : arr == 2 ? a.pv_s : a.pv_b) +
+                               row0 * 4 * kSB;
+      const int sb_half = kSB == 4 ? (wave >> 2) * 256 : 0;
+      const uint32_t code_off = (uint32_t)tid * 16;  // K / V codes: LDS slot tid of the tile's 512
+      const uint32_t sb_off = (uint32_t)(sb_half + lane * 4);
+      auto issue_raw = [&](int t, int rslot) {
+        if (t > p_end - 1) t = p_end - 1;  // past the end: a harmless re-read, so that the counts stay static
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0) + kRawBase + rslot * kRawBytes;
+        async_load_16((uint64_t)(kc + (int64_t)t * kCodeBytes), code_off, dst + wave * 1024);
+        async_load_16((uint64_t)(vc + (int64_t)t * kCodeBytes), code_off, dst + kCodeBytes + wave * 1024);
+        async_load_4((uint64_t)(sb_base + (int64_t)t * kScaleBytes), sb_off, dst + 2 * kCodeBytes + arr * 512 + sb_half);
       };
-      auto unpack_to = [&](int slot) {
+      auto unpack = [&](int rslot, int slot) {
+        // (the per-thread offsets are re-derived from the thread index at each use, which the empty asm
+        // enforces: carried across the loop they end up in scratch, and a reload waits behind the copies)
+        int tl = tid;
+        asm volatile("" : "+v"(tl));
+        const int row = tl >> 4, pp = tl & 15;  // tile row and its 16 elements [16 pp, +16), scale group pp / 4
+        const unsigned char* raw = lds + kRawBase + rslot * kRawBytes;
+        const u32x4_t rk = *reinterpret_cast<const u32x4_t*>(raw + tl * 16);
+        const u32x4_t rv = *reinterpret_cast<const u32x4_t*>(raw + kCodeBytes + tl * 16);
+        uint32_t rs[4];
+        const unsigned char* sp = raw + 2 * kCodeBytes + (row * 4 + (pp >> 2)) * kSB;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          if constexpr (SDT == MSPR_F32) rs[i] = *reinterpret_cast<const uint32_t*>(sp + i * 512);
+          else rs[i] = *reinterpret_cast<const uint16_t*>(sp + i * 512);
+        }
+        const int f = swz(row);
+        const int w_off0 = row * kRowBytes + 16 * (((2 * pp) & 16) | (((2 * pp) ^ f) & 15));
+        const int w_off1 = row * kRowBytes + 16 * (((2 * pp + 1) & 16) | (((2 * pp + 1) ^ f) & 15));
         unsigned char* st = lds + slot * kStageBytes;
         u32x4_t p0, p1;
         dequant16(rk, sb_to_h2<SDT>(rs[0]), sb_to_h2<SDT>(rs[1]), p0, p1);
@@ -381,18 +417,23 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
         *reinterpret_cast<u32x4_t*>(st + kTileBytes + w_off0) = p0;
         *reinterpret_cast<u32x4_t*>(st + kTileBytes + w_off1) = p1;
       };
-      load_raw(t_begin);
-      unpack_to(0);
-      if (t_begin + 1 < p_end) load_raw(t_begin + 1);
+      issue_raw(t_begin, 0);
+      issue_raw(t_begin + 1, 1);
+      issue_raw(t_begin + 2, 2);
+      wait_vm_and_barrier<6>();  // the raw bytes of the first tile are in LDS
+      unpack(0, 0);
       for (int t = t_begin; t < p_end; t++) {
-        __syncthreads();  // tile t is complete in LDS; every wave has left tile t-1
-        if (t + 1 < p_end) {
-          unpack_to((t + 1 - t_begin) & 1);
-          if (t + 2 < p_end) load_raw(t + 2);
-        }
-        compute_tile(lds + ((t - t_begin) & 1) * kStageBytes, t * kTile);
+        const int i = t - t_begin;
+        // this wave's copies of raw tile t+1 are done (those of t+2 may be in flight); after the barrier
+        // every wave's are, stage i & 1 holds tile t, and stage (i + 1) & 1 and raw slot i % 3 are free
+        wait_vm_and_barrier<3>();
+        issue_raw(t + 3, i % 3);
+        if (t + 1 < p_end) unpack((i + 1) % 3, (i + 1) & 1);
+        compute_tile(lds + (i & 1) * kStageBytes, t * kTile);
       }
-      __syncthreads();  // every wave has left the last prefix tile before the ring below reuses the slots
+      // every wave has left the last prefix tile and the trailing raw copies have landed before the ring
+      // below reuses the LDS
+      wait_vm_and_barrier<0>();
     }
   }
 
@@ -692,6 +733,10 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
                "sdpa_fa_prefill_q8: need q_len >= 1 and past_len >= 0");
   MSPR_REQUIRE(mspr_aligned(queries, 16) && mspr_aligned(out, 16) && mspr_aligned(pk_wq, 16) && mspr_aligned(pv_wq, 16),
                "sdpa_fa_prefill_q8: pointers must be 16-byte aligned");
+  // (scales and biases move to LDS four bytes per lane)
+  MSPR_REQUIRE(mspr_aligned(pk_scales, 4) && mspr_aligned(pk_biases, 4) && mspr_aligned(pv_scales, 4) &&
+                   mspr_aligned(pv_biases, 4),
+               "sdpa_fa_prefill_q8: scales and biases must be 4-byte aligned");
   const size_t need = mspr_sdpa_fa_prefill_q8_workspace_bytes(batch, n_q_heads, n_kv_heads, q_len, past_len);
   MSPR_REQUIRE(workspace && workspace_bytes >= need && mspr_aligned(workspace, 16),
                "sdpa_fa_prefill_q8: workspace of %zu bytes (16-byte aligned) needed, %zu given", need, workspace_bytes);
