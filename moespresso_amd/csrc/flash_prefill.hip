@@ -141,19 +141,33 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   const int n = lane & 31;  // MFMA column: query row of the wave's block; MFMA row (key) for the K operand
   const int g = lane >> 5;
 
-  // ---- workgroup -> (batch, kv head, query block); late blocks (most keys) first
+  // ---- workgroup -> (batch, kv head, pair of query row ranges, half of the heads when eight share a KV head).
+  // Waves 0-3 take 32-row blocks from the late end of the chunk (most keys), waves 4-7 the mirrored blocks from
+  // the early end, so every workgroup carries the same matrix work although the causal key count grows with the
+  // query position; the tile stream runs to the late block's last key and the early waves leave it when their
+  // last key has passed. Four heads per group; with fewer heads per KV head a group takes 2 or 4 adjacent blocks.
   const int rep = 1 << a.rep_shift;
-  const int sub_blocks = 8 >> a.rep_shift;  // 32-row query sub-blocks per workgroup
-  const int rows_per_wg = 32 * sub_blocks;
+  const int hpg_shift = a.rep_shift < 2 ? a.rep_shift : 2;  // log2(heads per group)
+  const int blocks_per_group = 4 >> hpg_shift;
+  const int head_halves = 1 << (a.rep_shift - hpg_shift);
+  const int n_blocks = (a.q_len + 31) / 32;
+  const int n_pairs = a.q_blocks / head_halves;
   int work = blockIdx.x;
   const int sp = work % a.n_splits;
   work /= a.n_splits;
-  const int qb = a.q_blocks - 1 - work % a.q_blocks;
+  const int pair = (work % a.q_blocks) / head_halves;  // pair 0 (longest stream) first
+  const int head_half = work % head_halves;
   work /= a.q_blocks;
   const int kvh = work % a.n_kv_heads;
   const int b = work / a.n_kv_heads;
-  const int head = kvh * rep + (wave & (rep - 1));
-  const int q0 = qb * rows_per_wg + 32 * (wave >> a.rep_shift);  // first query row of this wave
+  const int wi = wave & 3;
+  const int head = kvh * rep + (head_half << hpg_shift) + (wi & ((1 << hpg_shift) - 1));
+  // late group: blocks [n_blocks - bpg (pair + 1), n_blocks - bpg pair); early group: blocks [bpg pair, bpg (pair + 1))
+  // as far as they lie below the late groups' range [n_blocks - bpg n_pairs, n_blocks)
+  const int blk = wave < 4 ? n_blocks - blocks_per_group * (pair + 1) + (wi >> hpg_shift)
+                           : blocks_per_group * pair + (wi >> hpg_shift);
+  const bool active = wave < 4 ? blk >= 0 : blk < n_blocks - blocks_per_group * n_pairs;  // wave-uniform
+  const int q0 = active ? 32 * blk : 0;  // first query row of this wave
   const int past = (int)a.past_len;
 
   const unsigned char* kbase =
@@ -162,7 +176,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
       reinterpret_cast<const unsigned char*>(a.v) + ((int64_t)b * a.n_kv_heads + kvh) * a.kv_rows * kRowBytes;
 
   // keys needed by the workgroup: [0, past + last query row]
-  int q_last = qb * rows_per_wg + rows_per_wg - 1;
+  int q_last = 32 * (n_blocks - blocks_per_group * pair) - 1;  // last row of the late group
   if (q_last > a.q_len - 1) q_last = a.q_len - 1;
   const int all_tiles = (int)((past + q_last) / kTile) + 1;
   // this workgroup's share of the block's tiles: [t_begin, n_tiles)
@@ -242,7 +256,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
     const int r = tr_row + 8 * h;
     v_off[h] = kTileBytes + r * kRowBytes + 16 * ((tr_piece ^ swz(r)) & 15) + 8 * (tr_s & 1);
   }
-  const int my_last_key = past + q0 + 31;  // last key any query of this wave may see
+  const int my_last_key = active ? past + q0 + 31 : -1;  // last key any query of this wave may see
   const int qpos_g = past + q0 + n - 4 * g;  // the lane's query position minus its key offset inside a tile
 
   // stage 1 of a tile: S^T = K . Q^T on the matrix cores
@@ -429,7 +443,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
         wait_vm_and_barrier<3>();
         issue_raw(t + 3, i % 3);
         if (t + 1 < p_end) unpack((i + 1) % 3, (i + 1) & 1);
-        compute_tile(lds + (i & 1) * kStageBytes, t * kTile);
+        if (t * kTile <= my_last_key) compute_tile(lds + (i & 1) * kStageBytes, t * kTile);
       }
       // every wave has left the last prefix tile and the trailing raw copies have landed before the ring
       // below reuses the LDS
@@ -476,7 +490,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   // ---- normalise and store: lane (n, g) holds dims 32 mt + 8 (i/4) + 4 g + i%4 of query row q0 + n
   const float l_tot = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
   if (a.n_splits > 1) {
-    if (q0 + n < a.q_len) {
+    if (active && q0 + n < a.q_len) {
       const int64_t row = (((int64_t)sp * a.batch + b) * a.n_q_heads + head) * a.q_len + q0 + n;
       float* po = a.ws_o + row * kD;
 #pragma unroll
@@ -493,7 +507,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
     return;
   }
   const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
-  if (q0 + n < a.q_len) {
+  if (active && q0 + n < a.q_len) {
     const int64_t ooff = (((int64_t)b * a.n_q_heads + head) * a.q_len + q0 + n) * kD;
 #pragma unroll
     for (int mt = 0; mt < 8; mt++)
@@ -599,6 +613,16 @@ __global__ __launch_bounds__(256) void prefill_merge_kernel(PrefillArgs a) {
   }
 }
 
+// workgroups along the query axis: pairs of (late, early) row ranges, times two head halves when eight
+// query heads share a KV head (see the kernel's work mapping)
+int prefill_q_blocks(int rep, int q_len) {
+  const int heads_per_group = rep < 4 ? rep : 4;
+  const int blocks_per_group = 4 / heads_per_group;
+  const int n_blocks = (q_len + 31) / 32;
+  const int n_pairs = (n_blocks + 2 * blocks_per_group - 1) / (2 * blocks_per_group);
+  return n_pairs * (rep / heads_per_group);
+}
+
 // enough workgroups for the 256 CUs, at least 16 tiles (512 keys) per range
 int prefill_choose_splits(int batch, int n_kv_heads, int q_blocks, int64_t past_len, int q_len) {
   const int64_t wgs = (int64_t)batch * n_kv_heads * q_blocks;
@@ -612,8 +636,7 @@ int prefill_choose_splits(int batch, int n_kv_heads, int q_blocks, int64_t past_
 
 size_t prefill_split_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len, int64_t past_len) {
   const int rep = n_q_heads / n_kv_heads;
-  const int rows_per_wg = 32 * (8 / rep);
-  const int q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
+  const int q_blocks = prefill_q_blocks(rep, q_len);
   const int splits = prefill_choose_splits(batch, n_kv_heads, q_blocks, past_len, q_len);
   if (splits == 1) return 0;
   return (size_t)splits * batch * n_q_heads * q_len * (kD + 2) * sizeof(float);
@@ -685,8 +708,7 @@ extern "C" int mspr_flash_prefill(const void* q, const void* k, const void* v, i
   a.kv_rows = kv_rows;
   a.scale_log2 = (float)((double)scale * 1.4426950408889634);
   a.rep_shift = rep == 1 ? 0 : rep == 2 ? 1 : rep == 4 ? 2 : 3;
-  const int rows_per_wg = 32 * (8 / rep);
-  a.q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
+  a.q_blocks = prefill_q_blocks(rep, q_len);
   a.n_splits = prefill_choose_splits(batch, n_kv_heads, a.q_blocks, past_len, q_len);
   MSPR_REQUIRE((int64_t)a.q_blocks * n_kv_heads * batch * a.n_splits < ((int64_t)1 << 31), "flash_prefill: grid too large");
   if (a.n_splits > 1) {
@@ -756,8 +778,7 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
   a.kv_rows = tail_rows;
   a.scale_log2 = (float)((double)scale * 1.4426950408889634);
   a.rep_shift = rep == 1 ? 0 : rep == 2 ? 1 : rep == 4 ? 2 : 3;
-  const int rows_per_wg = 32 * (8 / rep);
-  a.q_blocks = (q_len + rows_per_wg - 1) / rows_per_wg;
+  a.q_blocks = prefill_q_blocks(rep, q_len);
   a.q8_tiles = (int)(past_len / kTile);
   a.n_splits = prefill_choose_splits(batch, n_kv_heads, a.q_blocks, past_len, q_len);
   if (a.n_splits > 1) {
