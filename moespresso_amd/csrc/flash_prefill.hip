@@ -1,9 +1,11 @@
 // Causal chunked-prefill GQA attention, head dim 256: a chunk of q_len new tokens attends to the
 // past_len tokens already in the KV cache and, causally, to itself.
 //
-// Workgroup = 8 waves = the query heads that share one KV head (times query sub-blocks when fewer
-// than 8 heads share it) x 32 query rows each, so one K/V tile staged in LDS feeds eight waves.
-// K/V tiles of 32 keys stream through a 3-deep LDS ring with asynchronous global->LDS copies; the
+// Workgroup = 8 waves on one KV head, 32 query rows per wave: two groups of four waves (four query
+// heads, or fewer heads times adjacent 32-row blocks), one group on a late block of the chunk and the
+// other on the mirrored early block, so one K/V tile staged in LDS feeds eight waves and every
+// workgroup carries the same matrix work under the causal mask.
+// K/V tiles of 32 keys stream through a 4-slot LDS ring with asynchronous global->LDS copies; the
 // 16-byte pieces of a row are XOR-swizzled on the way in (the copy writes LDS linearly, the global
 // address of each lane is free), which makes both the K operand reads (ds_read_b128, lane = key) and
 // the V^T operand reads (LDS transpose read) bank-conflict free without padding.
