@@ -98,52 +98,6 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
   const uint8_t* vc = reinterpret_cast<const uint8_t*>(a.v_codes) + kv_row0 * kD;
   constexpr int kGroups = FMT == kFmtQ8_0 ? 8 : 4;  // scale groups per row
 
-  // ---- Q^T operand: lane (n = head, g) holds q[head][64g + 8s .. +7] for k-step s, pre-multiplied by
-  //      scale * log2(e) and rounded to float16
-  u32x4_t qf[8];
-  {
-    const bool live = n < rep;
-    const int64_t qoff = ((int64_t)b * a.n_q_heads + kvh * rep + (live ? n : 0)) * kD + 64 * g;
-    float v[8][8];
-    if constexpr (QDT == MSPR_F32) {
-      const f32x4_t* p = reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(a.q) + qoff);
-      f32x4_t raw[16];
-#pragma unroll
-      for (int j = 0; j < 16; j++) raw[j] = p[j];
-#pragma unroll
-      for (int s = 0; s < 8; s++)
-#pragma unroll
-        for (int j = 0; j < 8; j++) v[s][j] = raw[2 * s + (j >> 2)][j & 3];
-    } else {
-      const u32x4_t* p = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(a.q) + qoff);
-      u32x4_t raw[8];
-#pragma unroll
-      for (int s = 0; s < 8; s++) raw[s] = p[s];
-#pragma unroll
-      for (int s = 0; s < 8; s++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-          if constexpr (QDT == MSPR_F16) {
-            v[s][2 * j] = f16_bits_to_f32((uint16_t)(raw[s][j] & 0xFFFFu));
-            v[s][2 * j + 1] = f16_bits_to_f32((uint16_t)(raw[s][j] >> 16));
-          } else {
-            v[s][2 * j] = bf16_bits_to_f32((uint16_t)(raw[s][j] & 0xFFFFu));
-            v[s][2 * j + 1] = bf16_bits_to_f32((uint16_t)(raw[s][j] >> 16));
-          }
-        }
-    }
-#pragma unroll
-    for (int s = 0; s < 8; s++) {
-      u32x4_t f;
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        h2_t h = {(_Float16)(live ? v[s][2 * j] * a.scale_log2 : 0.0f), (_Float16)(live ? v[s][2 * j + 1] * a.scale_log2 : 0.0f)};
-        f[j] = h2_bits(h);
-      }
-      qf[s] = f;
-    }
-  }
-
   f32x4_t oacc[16];
 #pragma unroll
   for (int mt = 0; mt < 16; mt++) oacc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -237,6 +191,55 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
     load_k(k0 + (int64_t)wave * kTileKeys);
     load_v(k0 + (int64_t)wave * kTileKeys);
   }
+  __builtin_amdgcn_sched_barrier(0);  // the first tile is on its way before the query is fetched: one memory
+                                      // round trip in front of the first MFMA instead of two
+
+  // ---- Q^T operand: lane (n = head, g) holds q[head][64g + 8s .. +7] for k-step s, pre-multiplied by
+  //      scale * log2(e) and rounded to float16
+  u32x4_t qf[8];
+  {
+    const bool live = n < rep;
+    const int64_t qoff = ((int64_t)b * a.n_q_heads + kvh * rep + (live ? n : 0)) * kD + 64 * g;
+    float v[8][8];
+    if constexpr (QDT == MSPR_F32) {
+      const f32x4_t* p = reinterpret_cast<const f32x4_t*>(reinterpret_cast<const float*>(a.q) + qoff);
+      f32x4_t raw[16];
+#pragma unroll
+      for (int j = 0; j < 16; j++) raw[j] = p[j];
+#pragma unroll
+      for (int s = 0; s < 8; s++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[s][j] = raw[2 * s + (j >> 2)][j & 3];
+    } else {
+      const u32x4_t* p = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(a.q) + qoff);
+      u32x4_t raw[8];
+#pragma unroll
+      for (int s = 0; s < 8; s++) raw[s] = p[s];
+#pragma unroll
+      for (int s = 0; s < 8; s++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          if constexpr (QDT == MSPR_F16) {
+            v[s][2 * j] = f16_bits_to_f32((uint16_t)(raw[s][j] & 0xFFFFu));
+            v[s][2 * j + 1] = f16_bits_to_f32((uint16_t)(raw[s][j] >> 16));
+          } else {
+            v[s][2 * j] = bf16_bits_to_f32((uint16_t)(raw[s][j] & 0xFFFFu));
+            v[s][2 * j + 1] = bf16_bits_to_f32((uint16_t)(raw[s][j] >> 16));
+          }
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      u32x4_t f;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        h2_t h = {(_Float16)(live ? v[s][2 * j] * a.scale_log2 : 0.0f), (_Float16)(live ? v[s][2 * j + 1] * a.scale_log2 : 0.0f)};
+        f[j] = h2_bits(h);
+      }
+      qf[s] = f;
+    }
+  }
+
   for (int64_t tile = wave; tile < n_tiles; tile += 4) {
     const int64_t key0 = k0 + tile * kTileKeys;
     const int64_t next_key0 = tile + 4 < n_tiles ? key0 + 4 * kTileKeys : key0;
@@ -422,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
       f32x4_t v = *reinterpret_cast<const f32x4_t*>(xo + ((w * 16 + mt) * 64 + lane) * 4);
       acc += v * mw[w];
     }
-    *reinterpret_cast<f32x4_t*>(po + n * kD + 16 * mt + 4 * g) = acc;
+    if (n < rep) *reinterpret_cast<f32x4_t*>(po + n * kD + 16 * mt + 4 * g) = acc;  // (columns past the real heads are padding)
   }
   if (wave == 0 && g == 0) {
     float* pml = a.ws_ml + part * 32;
@@ -432,13 +435,15 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
 }
 
 // Merge of the per-range partials: one workgroup per (batch, query head); 64 lanes cover the 256
-// dims four at a time, the 8 waves each take every 8th range, the wave results are combined in LDS.
+// dims four at a time, the 16 waves each take every 16th range and fetch up to 16 of them in one go
+// (one memory round trip for up to 256 ranges), the wave results are combined in LDS.
+constexpr int kMergeWaves = 16;
 template <int ODT>
-__global__ __launch_bounds__(512) void q8_decode_merge_kernel(Q8Args a) {
-  __shared__ float xm[8], xl[8];
-  __shared__ __attribute__((aligned(16))) float xo[8][kD];
+__global__ __launch_bounds__(64 * kMergeWaves) void q8_decode_merge_kernel(Q8Args a) {
+  __shared__ float xm[kMergeWaves], xl[kMergeWaves];
+  __shared__ __attribute__((aligned(16))) float xo[kMergeWaves][kD];
   const int lane = threadIdx.x & 63;
-  const int sg = threadIdx.x >> 6;
+  const int sg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int qh = blockIdx.x;
   const int b = blockIdx.y;
   const int rep = a.n_q_heads / a.n_kv_heads;
@@ -446,20 +451,23 @@ __global__ __launch_bounds__(512) void q8_decode_merge_kernel(Q8Args a) {
   const int64_t part0 = ((int64_t)b * a.n_kv_heads + kvh) * a.n_splits;
   const float* ml = a.ws_ml + part0 * 32 + hn * 2;
   const float* po = a.ws_o + part0 * (16 * kD) + hn * kD + 4 * lane;
-  constexpr int kChunk = 4;
+  constexpr int kChunk = 16;
   float m_run = -__builtin_inff(), l = 0.0f;
   f32x4_t o = {0.f, 0.f, 0.f, 0.f};
-  for (int s0 = sg; s0 < a.n_splits; s0 += 8 * kChunk) {
+  for (int s0 = sg; s0 < a.n_splits; s0 += kMergeWaves * kChunk) {
     float mv[kChunk], lv[kChunk];
     f32x4_t ov[kChunk];
 #pragma unroll
     for (int j = 0; j < kChunk; j++) {
-      const int sj = s0 + 8 * j;
-      const bool live = sj < a.n_splits;
-      const int64_t si = live ? sj : 0;
-      mv[j] = live ? ml[si * 32] : -__builtin_inff();
-      lv[j] = live ? ml[si * 32 + 1] : 0.0f;
-      ov[j] = *reinterpret_cast<const f32x4_t*>(po + si * (16 * kD));
+      const int sj = s0 + kMergeWaves * j;  // wave-uniform: ranges past the end cost no load
+      mv[j] = -__builtin_inff();
+      lv[j] = 0.0f;
+      ov[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (sj < a.n_splits) {
+        mv[j] = ml[(int64_t)sj * 32];
+        lv[j] = ml[(int64_t)sj * 32 + 1];
+        ov[j] = *reinterpret_cast<const f32x4_t*>(po + (int64_t)sj * (16 * kD));
+      }
     }
     float m_new = m_run;
 #pragma unroll
@@ -485,12 +493,12 @@ __global__ __launch_bounds__(512) void q8_decode_merge_kernel(Q8Args a) {
   if (sg != 0) return;
   float m_all = -__builtin_inff();
 #pragma unroll
-  for (int w = 0; w < 8; w++) m_all = fmaxf(m_all, xm[w]);
+  for (int w = 0; w < kMergeWaves; w++) m_all = fmaxf(m_all, xm[w]);
   const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
   float l_all = 0.0f;
   f32x4_t o_all = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int w = 0; w < 8; w++) {
+  for (int w = 0; w < kMergeWaves; w++) {
     const float wt = __builtin_amdgcn_exp2f(xm[w] - m_safe);
     l_all += xl[w] * wt;
     o_all += *reinterpret_cast<const f32x4_t*>(&xo[w][4 * lane]) * wt;
@@ -509,18 +517,28 @@ __global__ __launch_bounds__(512) void q8_decode_merge_kernel(Q8Args a) {
   }
 }
 
-int q8_choose_splits(int batch, int n_kv_heads, int64_t n_keys) {
-  // about two workgroups per CU, each with at least two tiles per wave
-  int64_t bh = (int64_t)batch * n_kv_heads;
-  int64_t want = (512 + bh - 1) / bh;
-  int64_t max_splits = (n_keys + 255) / 256;
-  if (want > max_splits) want = max_splits;
-  if (want < 1) want = 1;
-  return (int)want;
+// Key ranges: keys per range (whole 32-key tiles) and number of ranges. The split kernel's workgroups are
+// all resident at once and the memory system serves the CUs about evenly, so the launch ends with the CU
+// that holds the most tiles: a workgroup count just above the CU count (290 on 256 CUs) nearly doubles
+// the time of a short launch, and two workgroups on every CU measured slower than one with twice the
+// tiles (more partials, no more bandwidth). Hence at most one workgroup per CU, and never fewer than one
+// tile per wave in a range.
+void q8_plan(int batch, int n_kv_heads, int64_t n_keys, int64_t* keys_per_split, int* n_splits) {
+  const int64_t bh = (int64_t)batch * n_kv_heads;
+  const int64_t tiles = (n_keys + kTileKeys - 1) / kTileKeys;
+  int64_t ranges = 256 / bh;
+  if (ranges < 1) ranges = 1;
+  int64_t per = (tiles + ranges - 1) / ranges;
+  if (per < 4) per = 4;
+  *keys_per_split = per * kTileKeys;
+  *n_splits = (int)((tiles + per - 1) / per);
 }
 
 size_t q8_workspace_bytes(int batch, int n_kv_heads, int64_t n_keys) {
-  size_t parts = (size_t)batch * n_kv_heads * q8_choose_splits(batch, n_kv_heads, n_keys);
+  int64_t kps;
+  int splits;
+  q8_plan(batch, n_kv_heads, n_keys, &kps, &splits);
+  size_t parts = (size_t)batch * n_kv_heads * splits;
   return parts * (16 * kD + 32) * sizeof(float) + 256;
 }
 
@@ -546,7 +564,7 @@ int q8_launch(Q8Args a, hipStream_t st) {
   dim3 mgrid((unsigned)a.n_q_heads, (unsigned)a.batch);
   {
     MsprProfScope prof(MSPR_K_Q8_MERGE, st);
-    dim3 mblock(512);
+    dim3 mblock(64 * kMergeWaves);
     if (QDT == MSPR_F32) q8_decode_merge_kernel<MSPR_F32><<<mgrid, mblock, 0, st>>>(a);
     else if (QDT == MSPR_BF16) q8_decode_merge_kernel<MSPR_BF16><<<mgrid, mblock, 0, st>>>(a);
     else q8_decode_merge_kernel<MSPR_F16><<<mgrid, mblock, 0, st>>>(a);
@@ -578,11 +596,9 @@ void q8_fill_args(Q8Args& a, int batch, int n_q_heads, int n_kv_heads, int64_t n
   a.n_kv_heads = n_kv_heads;
   a.n_keys = n_keys;
   a.scale_log2 = (float)((double)scale * 1.4426950408889634);
-  const int want = q8_choose_splits(batch, n_kv_heads, n_keys);
-  int64_t kps = (n_keys + want - 1) / want;
-  kps = (kps + 127) / 128 * 128;  // whole tiles for all four waves
+  int64_t kps;
+  q8_plan(batch, n_kv_heads, n_keys, &kps, &a.n_splits);
   a.keys_per_split = (int)kps;
-  a.n_splits = (int)((n_keys + kps - 1) / kps);  // never more than `want`: the workspace bound holds
   size_t parts = (size_t)batch * n_kv_heads * a.n_splits;
   a.ws_o = reinterpret_cast<float*>(workspace);
   a.ws_ml = a.ws_o + parts * (16 * kD);

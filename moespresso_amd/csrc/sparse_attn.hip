@@ -760,11 +760,12 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
 }
 
 int choose_splits(int batch_hblk, int n_keys) {
-  // enough workgroups to cover the 256 CUs, at least one 32-slot tile each, and never more gathered
+  // enough workgroups to cover the 256 CUs but not one more (all are resident at once and a CU that holds
+  // two of them takes about twice as long), at least one 32-slot tile each, and never more gathered
   // slots per workgroup than its LDS id table holds
   int tiles = (n_keys + kTile - 1) / kTile;
   if (tiles < 1) tiles = 1;
-  int want = (256 + batch_hblk - 1) / batch_hblk;
+  int want = batch_hblk <= 256 ? 256 / batch_hblk : 1;
   if (want > 32) want = 32;
   if (want > tiles) want = tiles;
   int min_splits = (n_keys + 1023) / 1024;
