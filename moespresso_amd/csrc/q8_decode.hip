@@ -6,7 +6,7 @@
 //            bias per 64 elements (the MLX affine 8-bit layout)
 // Head dim 256, up to 16 query heads per KV head.
 //
-// A workgroup owns (batch, kv head, key range); each of its four waves walks 32-key tiles of that
+// A workgroup owns (batch, kv head, key range); each of its waves walks 32-key tiles of that
 // range on its own (private online softmax state), the waves are merged through LDS at the end and
 // the per-range partials by a second kernel.
 //
@@ -22,6 +22,7 @@ namespace {
 
 constexpr int kD = 256;
 constexpr int kTileKeys = 32;
+constexpr int kQ8Waves = 4;  // waves per workgroup of the split kernel (8 measured 7-25 % slower at batch 8 / 1)
 constexpr int kVPitch = kD * 2 + 16;           // bytes per key row of the float16 V tile
 constexpr int kVTileBytes = kTileKeys * kVPitch;
 constexpr int kFmtQ8_0 = 0;
@@ -75,7 +76,7 @@ __device__ __forceinline__ void codes4_to_h(uint32_t w, h2_t& lo, h2_t& hi) {
 }
 
 template <int FMT, int QDT, int SDT>
-__global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
+__global__ __launch_bounds__(64 * kQ8Waves, 1) void q8_decode_split_kernel(Q8Args a) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -240,9 +241,9 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
     }
   }
 
-  for (int64_t tile = wave; tile < n_tiles; tile += 4) {
+  for (int64_t tile = wave; tile < n_tiles; tile += kQ8Waves) {
     const int64_t key0 = k0 + tile * kTileKeys;
-    const int64_t next_key0 = tile + 4 < n_tiles ? key0 + 4 * kTileKeys : key0;
+    const int64_t next_key0 = tile + kQ8Waves < n_tiles ? key0 + kQ8Waves * kTileKeys : key0;
 
     // ---- S^T = K . Q^T for the two 16-key sub-tiles
     f32x4_t sacc[2];
@@ -383,13 +384,13 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
     __builtin_amdgcn_wave_barrier();
   }
 
-  // ---- merge the four waves through LDS (the V tiles are free now), write this range's partial
+  // ---- merge the waves through LDS (the V tiles are free now), write this range's partial
   float l_tot = l_run;
   l_tot += __shfl_xor(l_tot, 16, MSPR_WAVE);
   l_tot += __shfl_xor(l_tot, 32, MSPR_WAVE);
   __syncthreads();
-  float* xo = reinterpret_cast<float*>(lds);              // [4 waves][16 mt][4][64 lanes]
-  float* xml = xo + 4 * 16 * 4 * 64;                      // [4 waves][16 heads][2]
+  float* xo = reinterpret_cast<float*>(lds);              // [waves][16 mt][4][64 lanes]
+  float* xml = xo + kQ8Waves * 16 * 4 * 64;               // [waves][16 heads][2]
 #pragma unroll
   for (int mt = 0; mt < 16; mt++)
     *reinterpret_cast<f32x4_t*>(xo + ((wave * 16 + mt) * 64 + lane) * 4) = oacc[mt];
@@ -398,10 +399,10 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
     xml[(wave * 16 + n) * 2 + 1] = l_tot;
   }
   __syncthreads();
-  float mw[4], lw[4];
+  float mw[kQ8Waves], lw[kQ8Waves];
   float m_all = -__builtin_inff();
 #pragma unroll
-  for (int w = 0; w < 4; w++) {
+  for (int w = 0; w < kQ8Waves; w++) {
     mw[w] = xml[(w * 16 + n) * 2];
     lw[w] = xml[(w * 16 + n) * 2 + 1];
     m_all = fmaxf(m_all, mw[w]);
@@ -409,19 +410,19 @@ __global__ __launch_bounds__(256, 2) void q8_decode_split_kernel(Q8Args a) {
   const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
   float l_all = 0.0f;
 #pragma unroll
-  for (int w = 0; w < 4; w++) {
+  for (int w = 0; w < kQ8Waves; w++) {
     mw[w] = __builtin_amdgcn_exp2f(mw[w] - m_safe);
     l_all += lw[w] * mw[w];
   }
   const int64_t part = (((int64_t)b * a.n_kv_heads + kvh) * a.n_splits + sp);
   float* po = a.ws_o + part * (16 * kD);
-  // wave w reduces M-tiles 4w..4w+3: dims 16mt + 4g + i of head n
+  // every wave reduces its share of the 16 M-tiles: dims 16mt + 4g + i of head n
 #pragma unroll
-  for (int q4 = 0; q4 < 4; q4++) {
-    const int mt = wave * 4 + q4;
+  for (int q4 = 0; q4 < 16 / kQ8Waves; q4++) {
+    const int mt = wave * (16 / kQ8Waves) + q4;
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int w = 0; w < 4; w++) {
+    for (int w = 0; w < kQ8Waves; w++) {
       f32x4_t v = *reinterpret_cast<const f32x4_t*>(xo + ((w * 16 + mt) * 64 + lane) * 4);
       acc += v * mw[w];
     }
@@ -529,7 +530,7 @@ void q8_plan(int batch, int n_kv_heads, int64_t n_keys, int64_t* keys_per_split,
   int64_t ranges = 256 / bh;
   if (ranges < 1) ranges = 1;
   int64_t per = (tiles + ranges - 1) / ranges;
-  if (per < 4) per = 4;
+  if (per < kQ8Waves) per = kQ8Waves;
   *keys_per_split = per * kTileKeys;
   *n_splits = (int)((tiles + per - 1) / per);
 }
@@ -544,7 +545,8 @@ size_t q8_workspace_bytes(int batch, int n_kv_heads, int64_t n_keys) {
 
 template <int FMT, int QDT, int SDT>
 int q8_launch(Q8Args a, hipStream_t st) {
-  constexpr int kLds = 4 * kVTileBytes > (4 * 16 * 4 * 64 + 4 * 16 * 2) * 4 ? 4 * kVTileBytes : (4 * 16 * 4 * 64 + 4 * 16 * 2) * 4;
+  constexpr int kMergeLds = (kQ8Waves * 16 * 4 * 64 + kQ8Waves * 16 * 2) * 4;
+  constexpr int kLds = kQ8Waves * kVTileBytes > kMergeLds ? kQ8Waves * kVTileBytes : kMergeLds;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&q8_decode_split_kernel<FMT, QDT, SDT>),
@@ -555,7 +557,7 @@ int q8_launch(Q8Args a, hipStream_t st) {
     }
     attr_set = true;
   }
-  dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv_heads, (unsigned)a.batch), block(256);
+  dim3 grid((unsigned)a.n_splits, (unsigned)a.n_kv_heads, (unsigned)a.batch), block(64 * kQ8Waves);
   {
     MsprProfScope prof(MSPR_K_Q8_DECODE, st);
     q8_decode_split_kernel<FMT, QDT, SDT><<<grid, block, kLds, st>>>(a);
