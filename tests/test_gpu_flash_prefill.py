@@ -35,6 +35,11 @@ def _case(B, Hq, Hkv, L, past, dtype, seed, extra_rows=0):
     (1, 16, 2, 256, 2048, torch.bfloat16, 0),
     (1, 16, 2, 64, 4100, torch.bfloat16, 0),   # short chunk over a deep prefix: key-range splits + merge
     (1, 8, 2, 33, 3000, torch.float16, 7),
+    # odd numbers of 32-row blocks under the late/early pairing of blocks inside a workgroup
+    (1, 16, 2, 96, 40, torch.bfloat16, 0),     # 8 heads per KV head, 3 blocks
+    (1, 8, 2, 200, 17, torch.float16, 0),      # 4 heads per KV head, 7 blocks
+    (1, 4, 2, 150, 70, torch.bfloat16, 2),     # 2 heads per KV head, 5 blocks (two per group)
+    (1, 2, 2, 420, 5, torch.bfloat16, 0),      # 1 head per KV head, 14 blocks (four per group)
 ])
 def test_flash_prefill_matches_oracle(B, Hq, Hkv, L, past, dtype, extra):
     from moespresso_amd.runtime.qwen import kquant
@@ -50,6 +55,27 @@ def test_flash_prefill_matches_oracle(B, Hq, Hkv, L, past, dtype, extra):
         ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
         err = np.abs(got[b:b + 1].float().cpu().numpy() - want)
         assert (err <= 2e-3 + ulp * np.abs(want)).all(), err.max()
+
+
+def test_flash_prefill_full_size_sampled_rows():
+    """BASELINE config 2 at full size (4096 new tokens over a 32768-token prefix, 16 query / 2 KV heads):
+    sampled query rows (block boundaries, first, last) against the oracle run on that one row, 2e-3."""
+    from moespresso_amd.runtime.qwen import kquant
+
+    L, past, Hq, Hkv = 4096, 32768, 16, 2
+    g = torch.Generator().manual_seed(11)
+    q = (0.5 * torch.randn((1, Hq, L, 256), generator=g)).to(torch.bfloat16)
+    k = (0.5 * torch.randn((1, Hkv, past + L, 256), generator=g)).to(torch.bfloat16)
+    v = (0.5 * torch.randn((1, Hkv, past + L, 256), generator=g)).to(torch.bfloat16)
+    scale = 256 ** -0.5
+    got = kquant.flash_prefill(q.to(_dev()), k.to(_dev()), v.to(_dev()), scale, past_len=past).float().cpu().numpy()
+    kf, vf = k.float().numpy(), v.float().numpy()
+    for row in (0, 31, 32, 2047, 2048, 2079, 4064, 4095):
+        n = past + row + 1
+        want = qwen.causal_prefill_attention(q[:, :, row:row + 1].float().numpy(), kf[:, :, :n], vf[:, :, :n],
+                                             scale, past=past + row)
+        err = np.abs(got[:, :, row:row + 1] - want)
+        assert (err <= 2e-3 + 2.0 ** -8 * np.abs(want)).all(), (row, err.max())
 
 
 def test_flash_prefill_first_row_copies_v():
@@ -128,3 +154,30 @@ def test_sdpa_fa_prefill_q8_matches_oracle(past, L, sb_dtype, self_dtype):
     assert err < 1e-2, err
     # observed accuracy is far inside the bar: float16 staging of exactly representable code values
     assert err < 2e-3, err
+
+
+def test_sdpa_fa_prefill_q8_full_size_sampled_rows():
+    """The reference test's depth (4096 new tokens over a 32768-token 8-bit prefix): sampled query rows against
+    the oracle run on that one row over the dequantised prefix + chunk, 1e-2 (8-bit KV bar)."""
+    from moespresso_amd.runtime.qwen import kquant
+
+    L, past = 4096, 32768
+    q, kq8, vq8, sk, sv = _q8_inputs(past, L, seed=5, sb_dtype=torch.float32)
+    dev = _dev()
+
+    def words(w):
+        return torch.from_numpy(np.ascontiguousarray(w).view(np.int32)).to(dev).view(torch.uint32)
+
+    scale = 256 ** -0.5
+    got = kquant.sdpa_fa_prefill_q8(torch.from_numpy(q).to(dev), words(kq8[0]), kq8[1].to(dev), kq8[2].to(dev),
+                                    words(vq8[0]), vq8[1].to(dev), vq8[2].to(dev), torch.from_numpy(sk).to(dev),
+                                    torch.from_numpy(sv).to(dev), scale, bq=32, bk=16, stage=2).cpu().numpy()
+    k_all = np.concatenate([kq8[3], sk], axis=2)
+    v_all = np.concatenate([vq8[3], sv], axis=2)
+    for row in (0, 31, 32, 2048, 4095):
+        n = past + row + 1
+        want = qwen.causal_prefill_attention(q[:, :, row:row + 1], k_all[:, :, :n], v_all[:, :, :n], scale,
+                                             past=past + row)
+        err = np.abs(got[:, :, row:row + 1] - want).max()
+        assert err < 1e-2, (row, err)
+
