@@ -625,11 +625,12 @@ int prefill_q_blocks(int rep, int q_len) {
   return n_pairs * (rep / heads_per_group);
 }
 
-// enough workgroups for the 256 CUs, at least 16 tiles (512 keys) per range
+// enough workgroups for the 256 CUs but not more (one fits a CU, so a count just above 256 means a second
+// round for a few of them), at least 16 tiles (512 keys) per range
 int prefill_choose_splits(int batch, int n_kv_heads, int q_blocks, int64_t past_len, int q_len) {
   const int64_t wgs = (int64_t)batch * n_kv_heads * q_blocks;
   if (wgs >= 192) return 1;
-  int64_t want = (256 + wgs - 1) / wgs;
+  int64_t want = 256 / wgs;
   const int64_t tiles = (past_len + q_len + kTile - 1) / kTile;
   if (want > tiles / 16) want = tiles / 16;
   if (want > 32) want = 32;
