@@ -66,6 +66,8 @@ def test_sdpa_decode_q8_affine(B, Hq, Hkv, N, sb_dtype):
     (8, 37000, torch.bfloat16),
     (1, 513, torch.float16),
     (3, 2048, torch.float32),
+    (3, 37000, torch.bfloat16),   # batch x KV heads does not divide the CU count
+    (5, 9000, torch.float16),
 ])
 def test_sdpa_decode_q8_0(B, N, qdt):
     """BASELINE config 3: int8 codes + one float16 scale per 32, bf16 queries, batch 1 and 8."""
