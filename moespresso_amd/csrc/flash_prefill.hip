@@ -454,39 +454,29 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
   }
 
   // ---- dense tiles through the asynchronous ring: every wave issues its share of every tile
-  //      (clamped past the end), so the waits are static counts.
-  // The two waves that share a SIMD run half a tile apart: waves 4-7 (the early query blocks) do both
-  // stages of tile t in iteration t, waves 0-3 (the late blocks, which stay when the early ones have left
-  // the stream) do stage 2 of tile t-1 and then stage 1 of tile t, so that after the barrier the two are
-  // in different stages instead of queueing for the same unit (this assignment measured 2 % faster than
-  // the opposite one). The deferred group still reads tile t-1 in iteration t, hence four ring slots.
+  //      (clamped past the end), so the waits are static counts. Every wave runs both stages of tile t in
+  //      iteration t. (Running the two waves of a SIMD half a tile apart, one of them with stage 2 of tile
+  //      t-1 in front of stage 1 of tile t, paid while the tile loop still reloaded spilled registers; without
+  //      those reloads it measured 1.7 % slower than this order, and both waves deferred 5 % slower.)
+#ifndef MSPR_FP_TILES_AHEAD
+#define MSPR_FP_TILES_AHEAD 2
+#endif
+  constexpr int kTilesAhead = MSPR_FP_TILES_AHEAD;  // tiles in flight behind the one being consumed (at most kBufs - 1)
+  static_assert(kTilesAhead >= 1 && kTilesAhead <= kBufs - 1, "ring too small");
   const int r0 = t_begin > t1 ? t_begin : t1;  // first tile of this workgroup that is served from k / v
   if (r0 < n_tiles) {
-  issue_tile(r0, 0);
-  issue_tile(r0 + 1 < n_tiles ? r0 + 1 : n_tiles - 1, 1);
-  if (Q8 || wave >= 4) {  // (the quantised-prefix form keeps one schedule: its code is large enough already)
+#pragma unroll
+    for (int j = 0; j < kTilesAhead; j++) issue_tile(r0 + j < n_tiles ? r0 + j : n_tiles - 1, j);
     for (int t = r0; t < n_tiles; t++) {
-      // tile t has landed once this wave's copies of it are done (4 newer ones may be in flight) and
-      // every wave got here; the ring slot of tile t-2 is free after the barrier
-      wait_vm_and_barrier<4>();
-      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - r0 + 2) % kBufs);  // past the end: a harmless re-read
+      // tile t has landed once this wave's copies of it are done (those of the newer tiles may be in flight:
+      // four per tile) and every wave got here; the ring slot of tile t-1 is free after the barrier
+      wait_vm_and_barrier<4 * (kTilesAhead - 1)>();
+      issue_tile(t + kTilesAhead < n_tiles ? t + kTilesAhead : n_tiles - 1,
+                 (t - r0 + kTilesAhead) % kBufs);  // past the end: a harmless re-read
       const int key0 = t * kTile;
       if (key0 > my_last_key) continue;  // wave-uniform: this wave's queries see none of the tile
       compute_tile(lds + ((t - r0) % kBufs) * kStageBytes, key0);
     }
-  } else {
-    f32x16_t sacc;
-    bool pending = false;  // stage 2 of the previous tile still to do (wave-uniform)
-    for (int t = r0; t < n_tiles; t++) {
-      wait_vm_and_barrier<4>();
-      issue_tile(t + 2 < n_tiles ? t + 2 : n_tiles - 1, (t - r0 + 2) % kBufs);
-      if (pending) softmax_pv_tile(lds + ((t - 1 - r0) % kBufs) * kStageBytes, (t - 1) * kTile, sacc);
-      const int key0 = t * kTile;
-      pending = key0 <= my_last_key;
-      if (pending) qk_tile(lds + ((t - r0) % kBufs) * kStageBytes, sacc);
-    }
-    if (pending) softmax_pv_tile(lds + ((n_tiles - 1 - r0) % kBufs) * kStageBytes, (n_tiles - 1) * kTile, sacc);
-  }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped trailing copies must not outlive the workgroup's LDS
 
