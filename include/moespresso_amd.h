@@ -117,7 +117,7 @@ int mspr_indexer_scores_tiled_live(const void* q, const float* weights, const vo
 
 /* ------------------------------------------------------------------ DS4 sparse attention */
 
-/* Scratch bytes for the three gathered-attention entry points below. */
+/* Scratch bytes for the gathered-attention entry points below. */
 size_t mspr_sparse_attention_workspace_bytes(int batch, int n_heads, int64_t n_keys);
 
 /* One-token indexed mixed attention over a ring of raw rows plus gathered pool rows, K == V.

@@ -105,7 +105,6 @@ def sparse_attention_workspace(batch: int, n_heads: int, n_keys: int, device) ->
     return torch.empty((max(nbytes, 16) + 3) // 4, dtype=torch.float32, device=device)
 
 
-
 def q8_decode_workspace(batch: int, n_kv_heads: int, n_keys: int, device) -> torch.Tensor:
     """Scratch tensor for the Q8 decode entry points (per-range partials)."""
     nbytes = int(lib().mspr_sdpa_decode_q8_workspace_bytes(int(batch), int(n_kv_heads), int(n_keys)))

@@ -11,28 +11,19 @@
 // through LDS; for O^T = V^T.P^T it owns 128 of the 512 output columns. Two waves share a SIMD and
 // fill each other's waits (a wave has no matrix work while it stages or exchanges). V^T operands come
 // out of the same row-major tile through the LDS transpose read, so no second copy of the tile
-// exists. Partial (m, l, O) per slot range are merged by a second kernel (log-sum-exp), which also
-// applies the sink, the normalisation, the output cast and the optional inverse rope.
+// exists.
+//
+// Partial (m, l, O) per key range are merged by a second kernel (log-sum-exp), which also applies the
+// sink, the normalisation, the output cast and the optional inverse rope. (Merging inside the split
+// launch, behind a per-sequence arrival counter, was built and measured: the device-scope release of
+// the partials, the counter round trips and the partial reads are five dependent trips to memory of
+// about 2 us each at the end of every workgroup, against 6 us for the second launch.)
 //
 // MFMA shapes: v_mfma_f32_32x32x16_{f16,bf16}. Accumulator layout (lane l, register i):
 // column = l % 32, row = 8*(i/4) + 4*(l/32) + i%4. In S^T the column is the head and the row the
 // key, so softmax statistics are per lane; P^T registers feed the next MFMA's B operand unchanged.
 #include "common.h"
 #include "profile.h"
-
-#ifdef MSPR_SPARSE_TRACE
-// Debug build only: per-workgroup cycle stamps of the split kernel's phases.
-static long long* g_trace_buf = nullptr;
-extern "C" void mspr_debug_set_trace(long long* p) { g_trace_buf = p; }
-#define MSPR_STAMP(i)                                                         \
-  do {                                                                        \
-    if (a.trace && tid == 0) a.trace[(int64_t)blockIdx.x * 64 + (i)] = clock64(); \
-  } while (0)
-#else
-#define MSPR_STAMP(i) \
-  do {                \
-  } while (0)
-#endif
 
 namespace {
 
@@ -83,9 +74,11 @@ struct SparseAttnArgs {
   const float* inv_freq;
   const int32_t* params;
   int rope;
-  // split
+  // split: range sp of a sequence owns window slots [sp*win_per_split, +win_per_split) and gathered
+  // ids [sp*idx_per_split, +idx_per_split)
   int n_splits;
-  int slots_per_split;
+  int win_per_split;
+  int idx_per_split;
   int n_hblk;
   uint16_t* ws_o;  // float16 partial rows, each normalised by its own range's denominator
   float* ws_ml;
@@ -94,7 +87,6 @@ struct SparseAttnArgs {
   int out_dtype;
   int64_t out_batch_stride, out_head_stride, out_token_stride;  // elements
   int direct;  // one key range per sequence: the split kernel normalises and stores, no partials
-  long long* trace;  // debug builds only
 };
 
 template <int KDT>
@@ -225,7 +217,7 @@ struct Geometry {
   static constexpr int kSxBytes = 4 * 16 * 64 * 4; // 4 waves x 16 floats x 64 lanes (one head group)
   static constexpr int kMaxIds = 1024;             // gathered slots per workgroup
   static constexpr int kOffSx = kBufs * kTileBytes;
-  static constexpr int kMaxTiles = kMaxIds / kTile; // tiles per workgroup (slots_per_split <= kMaxIds)
+  static constexpr int kMaxTiles = kMaxIds / kTile; // tiles per workgroup
   static constexpr int kOffRowPtr = kOffSx + 2 * kSxBytes;       // row pointer of every slot of the workgroup
   static constexpr int kOffVmask = kOffRowPtr + kMaxIds * 8;     // one validity word per tile
   static constexpr int kOffRope = kOffVmask + kMaxTiles * 4;
@@ -284,17 +276,23 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     seq_visible = vis < a.n_pool ? vis : a.n_pool;
   }
 
-  const int n_keys = seq_n_win + a.n_idx;
-  const int slot0 = sp * a.slots_per_split;
-  int slot1 = slot0 + a.slots_per_split;
-  if (slot1 > n_keys) slot1 = n_keys;
-  const int n_tiles = slot1 > slot0 ? (slot1 - slot0 + kTile - 1) / kTile : 0;
+  // range sp: its share of the window slots, then its share of the gathered ids. Window tiles come
+  // first in the tile order: their rows need no ids, so their copies leave before the id round trip.
+  const int w0 = sp * a.win_per_split;
+  int w1 = w0 + a.win_per_split;
+  if (w1 > seq_n_win) w1 = seq_n_win;
+  const int wt = w1 > w0 ? (w1 - w0 + kTile - 1) / kTile : 0;
+  const int g0 = sp * a.idx_per_split;
+  int g1 = g0 + a.idx_per_split;
+  if (g1 > a.n_idx) g1 = a.n_idx;
+  const int gt = g1 > g0 ? (g1 - g0 + kTile - 1) / kTile : 0;
+  const int n_tiles = wt + gt;
+  const int g_ls0 = wt * kTile;  // first local slot of the gathered part
 
   const uint16_t* win_b = reinterpret_cast<const uint16_t*>(a.win) + (int64_t)b * a.win_batch_stride;
   const uint16_t* pool_b = reinterpret_cast<const uint16_t*>(a.pool) + (int64_t)b * a.pool_batch_stride;
   const int32_t* idx_b = a.idx + (int64_t)seq * a.idx_batch_stride;
 
-  MSPR_STAMP(0);
   // ---- query operand: lane (n = head, g) holds q[head][dh*kPart + 16ks + 8g .. +7]; its loads go out
   //      right behind the id loads below and are back by the time the row pointer table is built
   const int head = hb * 64 + hg * 32 + n;
@@ -304,12 +302,13 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   u32x4_t qf[G::kSteps];
   f32x4_t qraw32[QDT == MSPR_F32 ? G::kSteps : 1][2];
   // The gathered ids of this thread's slots are requested before anything else: ids -> row pointers ->
-  // rows is the longest dependency chain of the prologue. Slot ls = tid + 256 j of the range.
+  // rows is the longest dependency chain of the prologue. Local slot ls = tid + 512 j of the range.
   int my_id[G::kMaxIds / kThreads];
 #pragma unroll
   for (int j = 0; j < G::kMaxIds / kThreads; j++) {
-    const int gi = slot0 + tid + kThreads * j - seq_n_win;
-    my_id[j] = (gi >= 0 && gi < a.n_idx && j * kThreads < n_tiles * kTile) ? idx_b[gi] : -1;
+    const int ls = tid + kThreads * j;
+    const int gi = g0 + ls - g_ls0;
+    my_id[j] = (ls >= g_ls0 && gi < g1) ? idx_b[gi] : -1;
   }
   if constexpr (QDT == MSPR_F32) {
     const float* qp = reinterpret_cast<const float*>(a.q) + qoff;
@@ -324,28 +323,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = *reinterpret_cast<const u32x4_t*>(qp + 16 * ks);
   }
 
-
-  // ---- stop position of the gathered walk, rope table, gathered ids of this slot range
-  if (ROPE && tid < 32) {
-    float theta = (float)a.params[0] * a.inv_freq[tid];
-    rope_c[tid] = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
-    rope_s[tid] = f16_bits_to_f32(f32_to_f16_bits((float)sin((double)theta)));
-  }
-  int stop_pos = a.n_idx;
-  if (a.check_stop) {
-    if (tid == 0) *stop_shared = a.n_idx;
-    __syncthreads();
-    int first = a.n_idx;
-    for (int i = tid; i < a.n_idx; i += kThreads) {
-      int id = idx_b[i];
-      if (id >= 0 && (int64_t)id >= seq_visible && i < first) first = i;
-    }
-    if (first < a.n_idx) atomicMin(stop_shared, first);
-    __syncthreads();
-    stop_pos = *stop_shared;
-  }
-  const int subst_slot = a.subst_from_params ? a.params[1] : a.subst_slot;
-  // ---- static part of this thread's tile loads: LDS slot P = tid + 256 j holds (row P / kSlots, chunk P % kSlots)
+  // ---- static part of this thread's tile loads: LDS slot P = tid + 512 j holds (row P / kSlots, chunk P % kSlots)
   uint32_t pk[G::kPerThread];
 #pragma unroll
   for (int j = 0; j < G::kPerThread; j++) {
@@ -354,45 +332,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     pk[j] = (P < G::kTileSlots && chunk != G::kSlots - 1) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
   }
   const uint64_t zero_row = reinterpret_cast<uint64_t>(&g_zero_row[0]);
-
-  // ---- row pointer and validity of every slot of this workgroup's range, by all threads at once:
-  //      window slots map to ring rows (or the substituted row), gathered slots read their id from
-  //      global memory; skipped slots point at a zero row so that every tile load stays fully active
-#pragma unroll
-  for (int tj = 0; tj < G::kMaxIds / kThreads; tj++) {
-    const int s0 = tj * kThreads;
-    if (s0 >= n_tiles * kTile) break;
-    const int ls = s0 + tid;  // slot inside the range (the loop bound is a multiple of 32, whole waves or half waves run)
-    const int slot = slot0 + ls;
-    uint64_t ptr = zero_row;
-    bool valid = false;
-    if (slot < slot1) {
-      if (slot < seq_n_win) {
-        valid = true;
-        if (slot == subst_slot) {
-          ptr = reinterpret_cast<uint64_t>(a.subst_row);
-        } else {
-          uint32_t r = ((uint32_t)a.raw_start + (uint32_t)seq_win_first + (uint32_t)slot) % (uint32_t)a.raw_cap;
-          ptr = reinterpret_cast<uint64_t>(win_b + (int64_t)r * DK);
-        }
-      } else {
-        const int gi = slot - seq_n_win;  // index into the gathered id list
-        const int id = gi < stop_pos ? my_id[tj] : -1;
-        if (id >= 0) {
-          const int64_t r = (int64_t)id * a.row_mul + a.row_add;
-          if (r >= 0 && r < a.n_pool) {
-            valid = true;
-            ptr = reinterpret_cast<uint64_t>(pool_b + r * DK);
-          }
-        }
-      }
-    }
-    const uint64_t bal = __ballot(valid);
-    if (ls < n_tiles * kTile) {
-      rowptr[ls] = ptr;
-      if ((lane & 31) == 0) vmask[ls >> 5] = (uint32_t)(bal >> (lane & 32));
-    }
-  }
   // asynchronous loads of one tile straight into its LDS ring buffer: source addresses first (LDS
   // reads of the row pointers), then one 1 KB copy per call of issue_one
   auto tile_sources = [&](int tile, uint64_t (&src)[G::kPerThread]) {
@@ -420,10 +359,83 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     for (int j = 0; j < G::kPerThread; j++) issue_one(src, dst_lds, j);
   };
 
-  MSPR_STAMP(1);
+  // ---- row pointer and validity of the window slots (ring rows, or the substituted row); skipped slots
+  //      point at a zero row so that every tile load stays fully active. The first window tiles are
+  //      requested at once.
+  if (wt > 0) {
+    const int subst_slot = a.subst_from_params ? a.params[1] : a.subst_slot;
+#pragma unroll
+    for (int tj = 0; tj < G::kMaxIds / kThreads; tj++) {
+      if (tj * kThreads >= g_ls0) break;
+      const int ls = tj * kThreads + tid;  // (the bound is a multiple of 32: whole waves or half waves run)
+      const int slot = w0 + ls;
+      const bool valid = ls < g_ls0 && slot < w1;
+      uint64_t ptr = zero_row;
+      if (valid) {
+        if (slot == subst_slot) {
+          ptr = reinterpret_cast<uint64_t>(a.subst_row);
+        } else {
+          uint32_t r = ((uint32_t)a.raw_start + (uint32_t)seq_win_first + (uint32_t)slot) % (uint32_t)a.raw_cap;
+          ptr = reinterpret_cast<uint64_t>(win_b + (int64_t)r * DK);
+        }
+      }
+      const uint64_t bal = __ballot(valid);
+      if (ls < g_ls0) {
+        rowptr[ls] = ptr;
+        if ((lane & 31) == 0) vmask[ls >> 5] = (uint32_t)(bal >> (lane & 32));
+      }
+    }
+    lds_barrier();
+    issue_tile(0);
+    if (wt > 1) issue_tile(1);
+  }
+
+  // ---- stop position of the gathered walk, rope table
+  if (ROPE && tid < 32) {
+    float theta = (float)a.params[0] * a.inv_freq[tid];
+    rope_c[tid] = f16_bits_to_f32(f32_to_f16_bits((float)cos((double)theta)));
+    rope_s[tid] = f16_bits_to_f32(f32_to_f16_bits((float)sin((double)theta)));
+  }
+  int stop_pos = a.n_idx;
+  if (a.check_stop) {
+    if (tid == 0) *stop_shared = a.n_idx;
+    __syncthreads();
+    int first = a.n_idx;
+    for (int i = tid; i < a.n_idx; i += kThreads) {
+      int id = idx_b[i];
+      if (id >= 0 && (int64_t)id >= seq_visible && i < first) first = i;
+    }
+    if (first < a.n_idx) atomicMin(stop_shared, first);
+    __syncthreads();
+    stop_pos = *stop_shared;
+  }
+
+  // ---- row pointer and validity of the gathered slots, by all threads at once
+#pragma unroll
+  for (int tj = 0; tj < G::kMaxIds / kThreads; tj++) {
+    if (tj * kThreads >= n_tiles * kTile) break;
+    const int ls = tj * kThreads + tid;
+    const int gi = g0 + ls - g_ls0;  // index into the gathered id list
+    uint64_t ptr = zero_row;
+    bool valid = false;
+    if (ls >= g_ls0 && gi < g1) {
+      const int id = gi < stop_pos ? my_id[tj] : -1;
+      if (id >= 0) {
+        const int64_t r = (int64_t)id * a.row_mul + a.row_add;
+        if (r >= 0 && r < a.n_pool) {
+          valid = true;
+          ptr = reinterpret_cast<uint64_t>(pool_b + r * DK);
+        }
+      }
+    }
+    const uint64_t bal = __ballot(valid);
+    if (ls >= g_ls0 && ls < n_tiles * kTile) {
+      rowptr[ls] = ptr;
+      if ((lane & 31) == 0) vmask[ls >> 5] = (uint32_t)(bal >> (lane & 32));
+    }
+  }
   __syncthreads();  // row pointer table visible
-  MSPR_STAMP(61);
-  // The query loads (issued long ago) must be complete before the first asynchronous tile load goes
+  // The query loads (issued long ago) must be complete before the next asynchronous tile load goes
   // out: a wait left for their first use would otherwise also wait for (drain) the tile loads behind them.
   if constexpr (QDT == MSPR_F32) {
 #pragma unroll
@@ -432,10 +444,9 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 #pragma unroll
     for (int ks = 0; ks < G::kSteps; ks++) asm volatile("" : "+v"(qf[ks]));
   }
-  MSPR_STAMP(60);
-  if (n_tiles > 0) issue_tile(0);
-  if (n_tiles > 1) issue_tile(1);
-  MSPR_STAMP(2);
+  // two tiles are in flight when the tile loop starts
+  if (wt < 1 && n_tiles > 0) issue_tile(0);
+  if (wt < 2 && n_tiles > 1) issue_tile(1);
 
   // ---- finish the query operand (type conversion, rope) while the first tiles are in flight
   if constexpr (QDT == kQSame && !ROPE) {
@@ -476,7 +487,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
                       : u32x4_t{0u, 0u, 0u, 0u};
     }
   }
-  MSPR_STAMP(3);
 
   f32x16_t oacc[4];
 #pragma unroll
@@ -511,12 +521,10 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     } else {
       wait_vm_and_barrier<0>();
     }
-    MSPR_STAMP(4 + 6 * t);
     const int buf = t % G::kBufs;
     const unsigned char* kt = kbuf + buf * G::kTileBytes;
     const uint32_t mask_all = vmask[t];
 
-    MSPR_STAMP(5 + 6 * t);
     // S^T partial over this wave's half of the row width
     // (two accumulators, even and odd k-steps: a single chain of dependent MFMAs runs about a tenth
     // below the issue rate of independent ones)
@@ -553,9 +561,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     for (int c = 0; c < 4; c++)
       *reinterpret_cast<f32x4_t*>(sxw + (c * 64 + lane) * 4) =
           f32x4_t{sacc[4 * c], sacc[4 * c + 1], sacc[4 * c + 2], sacc[4 * c + 3]};
-    MSPR_STAMP(6 + 6 * t);
     lds_barrier();
-    MSPR_STAMP(7 + 6 * t);
     {
       const float* sxp = sx + (hg * 4) * (16 * 64);
       f32x4_t part[4][4];
@@ -620,7 +626,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       pf[ks] = u32x4_t{pack2<KDT>(sacc[8 * ks], sacc[8 * ks + 1]), pack2<KDT>(sacc[8 * ks + 2], sacc[8 * ks + 3]),
                        pack2<KDT>(sacc[8 * ks + 4], sacc[8 * ks + 5]), pack2<KDT>(sacc[8 * ks + 6], sacc[8 * ks + 7])};
 
-    MSPR_STAMP(8 + 6 * t);
     // O^T += V^T . P^T ; V^T operands through the LDS transpose read of the row-major tile
     // (k-step outer, output tile inner: consecutive MFMAs never share an accumulator)
 #pragma unroll
@@ -636,7 +641,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     }
   }
 
-  MSPR_STAMP(4 + 6 * n_tiles);
   float l_tot = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
   if (a.direct) {
     // ---- the only key range of this sequence: sink, normalise, store
@@ -692,7 +696,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
     ml[0] = m_run;
     ml[1] = l_tot;
   }
-  MSPR_STAMP(5 + 6 * n_tiles);
+
 }
 
 // Merge of the per-split partials: one workgroup per (batch, head block, wave slot, 32-column tile).
@@ -701,9 +705,13 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int c = tid >> 6;  // accumulator quad: registers 4c..4c+3 (half of a stored group of 8)
-  const int mt = blockIdx.x & 3;
-  const int wave = (blockIdx.x >> 2) & 7;  // wave of the split kernel whose registers this workgroup merges
-  const int bh = blockIdx.x >> 5;
+  // a sequence's partials are merged on the XCD whose workgroups wrote them (the split kernel's mapping), so
+  // that they are read from that XCD's L2
+  unsigned work = blockIdx.x;
+  if ((gridDim.x & 7u) == 0u) work = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const int mt = work & 3;
+  const int wave = (work >> 2) & 7;  // wave of the split kernel whose registers this workgroup merges
+  const int bh = work >> 5;
   const int hb = bh % a.n_hblk;
   const int seq = bh / a.n_hblk;
   const int b = seq / a.n_tokens;
@@ -761,25 +769,29 @@ __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a
 
 int choose_splits(int batch_hblk, int n_keys) {
   // enough workgroups to cover the 256 CUs but not one more (all are resident at once and a CU that holds
-  // two of them takes about twice as long), at least one 32-slot tile each, and never more gathered
-  // slots per workgroup than its LDS id table holds
+  // two of them takes about twice as long), at least one 32-slot tile each, and never more slots per
+  // workgroup than its LDS row pointer table holds (its window share and its gathered share are each
+  // padded to whole tiles: at most 62 slots of padding and 2 of rounding on top of n_keys / splits)
   int tiles = (n_keys + kTile - 1) / kTile;
   if (tiles < 1) tiles = 1;
   int want = batch_hblk <= 256 ? 256 / batch_hblk : 1;
   if (want > 32) want = 32;
   if (want > tiles) want = tiles;
-  int min_splits = (n_keys + 1023) / 1024;
+  int min_splits = (n_keys + 959) / 960;
   if (want < min_splits) want = min_splits;
   if (want < 1) want = 1;
   return want;
 }
+
+constexpr size_t kPartialBytes = 4 * 8 * 16 * 64 * sizeof(uint16_t);  // 64 heads x 512 columns, float16
+constexpr size_t kStatBytes = 64 * 2 * sizeof(float);                 // (m, l) per head
 
 size_t workspace_bytes(int batch, int n_heads, int64_t n_keys) {
   int n_hblk = (n_heads + 63) / 64;
   int splits = choose_splits(batch * n_hblk, (int)n_keys);
   if (splits == 1) return 256;  // one key range per sequence: stored directly, no partials
   size_t parts = (size_t)batch * n_hblk * splits;
-  return parts * (4 * 8 * 16 * 64 * sizeof(uint16_t)) + parts * 64 * 2 * sizeof(float) + 256;
+  return parts * (kPartialBytes + kStatBytes);
 }
 
 template <int KDT, int DK, int QDT, bool ROPE>
@@ -815,12 +827,10 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   }
   a.n_hblk = (a.n_heads + 63) / 64;
   a.n_splits = choose_splits(a.batch * a.n_hblk, n_keys);
-  int sps = (n_keys + a.n_splits - 1) / a.n_splits;
-  sps = (sps + 7) / 8 * 8;
-  if (sps < 8) sps = 8;
-  if (sps > 1024) sps = 1024;
-  a.slots_per_split = sps;
-  MSPR_REQUIRE((int64_t)sps * a.n_splits >= n_keys, "sparse attention: too many key slots (%d)", n_keys);
+  a.win_per_split = (a.n_win + a.n_splits - 1) / a.n_splits;
+  a.idx_per_split = (a.n_idx + a.n_splits - 1) / a.n_splits;
+  const int table_slots = (a.win_per_split + kTile - 1) / kTile * kTile + (a.idx_per_split + kTile - 1) / kTile * kTile;
+  MSPR_REQUIRE(table_slots <= 1024, "sparse attention: too many key slots (%d)", n_keys);
   a.direct = a.n_splits == 1;
   size_t need = workspace_bytes(a.batch, a.n_heads, n_keys);
   MSPR_REQUIRE(workspace && workspace_bytes_given >= need, "sparse attention: workspace of %zu bytes needed, %zu given",
@@ -828,10 +838,7 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   MSPR_REQUIRE(mspr_aligned(workspace, 16), "sparse attention: workspace must be 16-byte aligned");
   size_t parts = (size_t)a.batch * a.n_hblk * a.n_splits;
   a.ws_o = reinterpret_cast<uint16_t*>(workspace);
-  a.ws_ml = reinterpret_cast<float*>(a.ws_o + parts * (4 * 8 * 16 * 64));
-#ifdef MSPR_SPARSE_TRACE
-  a.trace = g_trace_buf;
-#endif
+  a.ws_ml = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(workspace) + parts * kPartialBytes);
   int rc;
   if (a.rope) rc = launch_split<MSPR_F16, 512, kQSame, true>(a, st);
   else if (a.q_dtype == MSPR_F32) rc = launch_split<MSPR_F16, 512, MSPR_F32, false>(a, st);
@@ -956,11 +963,10 @@ extern "C" int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* wi
   return run_sparse_attention(a, MSPR_F16, 512, workspace, workspace_bytes_given, (hipStream_t)stream);
 }
 
-extern "C" int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, const float* sinks,
-                                      int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
-                                      int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
-                                      float scale, void* out, void* workspace, size_t workspace_bytes_given,
-                                      void* stream) {
+static int sparse_mla_decode_impl(const void* q, const void* kv, const int32_t* rows, const float* sinks, int dtype,
+                                 int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool, int n_rows, int row_mul,
+                                 int row_add, int64_t win_start, int win_rows, float scale, void* out,
+                                 void* workspace, size_t workspace_bytes_given, void* stream) {
   MSPR_REQUIRE(q && kv && out, "sparse_mla_decode: null pointer");
   MSPR_REQUIRE(n_rows == 0 || rows, "sparse_mla_decode: null rows");
   MSPR_REQUIRE(dtype == MSPR_F16 || dtype == MSPR_BF16, "sparse_mla_decode: dtype must be f16 or bf16");
@@ -1074,4 +1080,13 @@ extern "C" int mspr_indexed_mixed_attention_prefill(const void* q, int q_dtype, 
   a.out_head_stride = q_head_stride;
   a.out_token_stride = q_token_stride;
   return run_sparse_attention(a, MSPR_F16, 512, workspace, workspace_bytes_given, (hipStream_t)stream);
+}
+
+extern "C" int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, const float* sinks,
+                                      int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
+                                      int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
+                                      float scale, void* out, void* workspace, size_t workspace_bytes_given,
+                                      void* stream) {
+  return sparse_mla_decode_impl(q, kv, rows, sinks, dtype, batch, n_heads, k_dim, v_dim, n_pool, n_rows, row_mul,
+                                row_add, win_start, win_rows, scale, out, workspace, workspace_bytes_given, stream);
 }

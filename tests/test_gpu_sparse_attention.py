@@ -169,11 +169,78 @@ def test_sparse_mla_decode_full_config_batch16_with_sinks():
     assert err < 2e-3, err
 
 
+def _mla_case(B, H, DK, N, R, W, seed, sinks=False, big_v=False):
+    gen = torch.Generator(device=dev()).manual_seed(seed)
+    kv = torch.randn((B, N, DK), device=dev(), generator=gen, dtype=torch.float32)
+    if big_v:
+        # columns 64..511 within +-6e4: every convex combination of them fits float16; columns 0..63 at 7e4 and
+        # beyond: every convex combination of them exceeds the float16 range
+        kv[..., 64:512] = (torch.rand((B, N, 448), device=dev(), generator=gen) * 2.0 - 1.0) * 6.0e4
+        kv[..., :64] = kv[..., :64].abs() * 3.0e4 + 7.0e4
+    kv = kv.to(torch.bfloat16)
+    q = torch.randn((B, H, DK), device=dev(), generator=gen).to(torch.bfloat16)
+    if big_v:
+        q = (q.float() * 1.0e-4).to(torch.bfloat16)   # keeps the logits of the huge rows moderate
+    rng = np.random.default_rng(seed)
+    ids = np.stack([np.sort(rng.choice((N - W) // 4, R, replace=False)) for _ in range(B)]).astype(np.int32)
+    snk = rng.standard_normal(H).astype(np.float32) if sinks else None
+    return q, kv, ids, snk
+
+
+def _mla_oracle(q, kv, ids, snk, W):
+    B, N, DK = kv.shape
+    rows = 4 * ids + 3
+    all_rows = np.concatenate([np.tile(np.arange(N - W, N, dtype=np.int32), (B, 1)), rows], axis=1)
+    gathered = np.stack([kv[b][torch.from_numpy(all_rows[b]).to(dev()).long()].float().cpu().numpy() for b in range(B)])
+    local = np.tile(np.arange(all_rows.shape[1]), (B, 1))
+    return ds4.sparse_mla_decode(q.float().cpu().numpy(), gathered, local, scale=DK ** -0.5, sinks=snk)
+
+
+def test_sparse_mla_decode_full_config_batch4():
+    # BASELINE config 5, batch 4 leg at full size (32 key ranges per sequence)
+    q, kv, ids, snk = _mla_case(4, 64, 576, 131072, 2048, 128, seed=4)
+    got = iak.sparse_mla_decode(q, kv, to_dev(ids), scale=576 ** -0.5, window_start=131072 - 128, window_rows=128,
+                                row_mul=4, row_add=3)
+    want = _mla_oracle(q, kv, ids, snk, 128)
+    err = np.abs(got.float().cpu().numpy() - want).max()
+    assert err < 2e-3, err
+
+
+def test_sparse_mla_decode_workspace_serves_calls_of_other_shapes():
+    # one workspace, sized for the largest call, reused by smaller ones (other range counts)
+    from moespresso_amd import _lib
+    q, kv, ids, snk = _mla_case(16, 64, 576, 8192, 500, 128, seed=11, sinks=True)
+    ws = _lib.sparse_attention_workspace(16, 64, 2048 + 128, dev())
+    kw = dict(scale=576 ** -0.5, window_start=8192 - 128, window_rows=128, sinks=to_dev(snk), row_mul=4, row_add=3)
+    base = iak.sparse_mla_decode(q, kv, to_dev(ids), workspace=ws, **kw)
+    assert np.abs(base.float().cpu().numpy() - _mla_oracle(q, kv, ids, snk, 128)).max() < 2e-3
+    sub = iak.sparse_mla_decode(q[:3], kv[:3], to_dev(ids[:3, :77]), workspace=ws, **kw)
+    assert np.abs(sub.float().cpu().numpy() - _mla_oracle(q[:3], kv[:3], ids[:3, :77], snk, 128)).max() < 4e-3
+    assert torch.equal(iak.sparse_mla_decode(q, kv, to_dev(ids), workspace=ws, **kw), base)
+
+
+def test_sparse_mla_decode_bf16_values_beyond_float16_range():
+    # Per-range partial rows are stored as float16 and saturate at +-65504 (a row list served by one key
+    # range is stored directly and not clamped). This pins the documented limit: columns whose V values
+    # all fit float16 stay within tolerance next to columns that do not, and those come out clamped at
+    # the float16 range rather than as inf/NaN.
+    q, kv, ids, snk = _mla_case(2, 64, 576, 4096, 300, 128, seed=3, big_v=True)
+    got = iak.sparse_mla_decode(q, kv, to_dev(ids), scale=576 ** -0.5, window_start=4096 - 128, window_rows=128,
+                                row_mul=4, row_add=3).float().cpu().numpy()
+    want = _mla_oracle(q, kv, ids, snk, 128)
+    assert np.isfinite(got).all()
+    # bf16 rounding of the output plus float16 rounding of partial rows with values up to 6e4
+    bound = 2.0 ** -7 * np.abs(want) + 2.0 ** -10 * 6.0e4
+    assert (np.abs(got - want)[..., 64:] <= bound[..., 64:]).all(), (np.abs(got - want) - bound)[..., 64:].max()
+    assert (want[..., :64] >= 7.0e4).all()
+    assert (got[..., :64] == 65536.0).all()      # 65504 rounded to bfloat16
+
+
 # (the last three take the two-tiles-per-unit form of the kernel: an odd tile count, a ragged last tile,
 # a ragged first half of the last unit)
 @pytest.mark.parametrize("cfg", [dict(B=1, H=64, N=1000), dict(B=3, H=64, N=4099), dict(B=2, H=20, N=64),
                                  dict(B=16, H=64, N=32768), dict(B=16, H=64, N=16416), dict(B=20, H=33, N=13123),
-                                 dict(B=32, H=64, N=8209)])
+                                 dict(B=32, H=64, N=8209), dict(B=1, H=64, N=32768)])
 def test_indexer_scores_fp8_and_topk(cfg):
     B, H, N = cfg["B"], cfg["H"], cfg["N"]
     rng = np.random.default_rng(B * 1000 + N)
