@@ -178,6 +178,20 @@ int mspr_sparse_mla_decode(const void* q, const void* kv, const int32_t* rows, c
                            int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
                            float scale, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* mspr_sparse_mla_decode without a workspace argument and without any allocation, for callers that
+ * cannot allocate: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * No counterpart in the reference. The per-range partials live in a scratch array that is
+ * part of the library's device image (mspr_sparse_mla_decode_static_max_bytes() = 16,908,288 bytes, held
+ * by every GPU the library runs on until the process ends), which bounds the call to 256 key ranges:
+ * every shape with batch * ceil(n_heads/64) <= 256 whose rows fit 960 per range (batch 16 at 2176 rows,
+ * batch 256 at 960) is accepted, anything larger is rejected with MSPR_ERR_ARG before any launch.
+ * All calls on one GPU share the array: calls that overlap on a GPU (two streams, two threads) race. */
+int mspr_sparse_mla_decode_static(const void* q, const void* kv, const int32_t* rows, const float* sinks,
+                                  int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
+                                  int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
+                                  float scale, void* out, void* stream);
+size_t mspr_sparse_mla_decode_static_max_bytes(void);
+
 /* Partial rotary embedding of the last 64 channels of rows laid out [n_outer, seq_len, width]
  * (interleaved pairs); the leading channels copy through.
  * Replaces fused_partial_rope, runtime/deepseek_v4/attention_seam_kernel.py:247 (the composed

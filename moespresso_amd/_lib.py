@@ -53,6 +53,10 @@ SIGNATURES = {
     "mspr_sparse_mla_decode": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int64, c_int,
                 c_int, c_int, c_int64, c_int, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "mspr_sparse_mla_decode_static": (
+        c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int64, c_int,
+                c_int, c_int, c_int64, c_int, c_float, c_void_p, c_void_p]),
+    "mspr_sparse_mla_decode_static_max_bytes": (c_size_t, []),
     "mspr_fused_partial_rope": (
         c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p]),
     "mspr_affine_q8_quantize": (

@@ -25,6 +25,13 @@
 #include "common.h"
 #include "profile.h"
 
+// Scratch of mspr_sparse_mla_decode_static, the entry point that allocates nothing: the partials of up to 256
+// key ranges (a grid of one workgroup per CU), 64 heads x 512 float16 and 64 x (m, l) float32 each. Every range
+// of a call is written before it is read, so nothing in it has to start at zero. Host code never uses this
+// name as an address: it asks for the device address once per device (static_scratch below).
+constexpr size_t kStaticBytes = 256 * (size_t)(64 * 512 * 2 + 64 * 2 * 4);
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
 namespace {
 
 constexpr int kTile = 32;
@@ -785,6 +792,7 @@ int choose_splits(int batch_hblk, int n_keys) {
 
 constexpr size_t kPartialBytes = 4 * 8 * 16 * 64 * sizeof(uint16_t);  // 64 heads x 512 columns, float16
 constexpr size_t kStatBytes = 64 * 2 * sizeof(float);                 // (m, l) per head
+static_assert(kStaticBytes == 256 * (kPartialBytes + kStatBytes), "static scratch: 256 key ranges");
 
 size_t workspace_bytes(int batch, int n_heads, int64_t n_keys) {
   int n_hblk = (n_heads + 63) / 64;
@@ -792,6 +800,32 @@ size_t workspace_bytes(int batch, int n_heads, int64_t n_keys) {
   if (splits == 1) return 256;  // one key range per sequence: stored directly, no partials
   size_t parts = (size_t)batch * n_hblk * splits;
   return parts * (kPartialBytes + kStatBytes);
+}
+
+// Address of the static scratch on the current device, looked up once per device (each GPU holds its own
+// copy of the array at its own address; the array's name is never used as an address in host code).
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    mspr_set_error("sparse attention: cannot identify the current device (%s)", hipGetErrorString(e));
+    return MSPR_ERR_LAUNCH;
+  }
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      mspr_set_error("sparse attention: no address for the static scratch on device %d (%s)", dev,
+                     hipGetErrorString(e));
+      return MSPR_ERR_LAUNCH;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return MSPR_OK;
 }
 
 template <int KDT, int DK, int QDT, bool ROPE>
@@ -1089,4 +1123,23 @@ extern "C" int mspr_sparse_mla_decode(const void* q, const void* kv, const int32
                                       void* stream) {
   return sparse_mla_decode_impl(q, kv, rows, sinks, dtype, batch, n_heads, k_dim, v_dim, n_pool, n_rows, row_mul,
                                 row_add, win_start, win_rows, scale, out, workspace, workspace_bytes_given, stream);
+}
+
+extern "C" size_t mspr_sparse_mla_decode_static_max_bytes(void) { return kStaticBytes; }
+
+extern "C" int mspr_sparse_mla_decode_static(const void* q, const void* kv, const int32_t* rows, const float* sinks,
+                                             int dtype, int batch, int n_heads, int k_dim, int v_dim, int64_t n_pool,
+                                             int n_rows, int row_mul, int row_add, int64_t win_start, int win_rows,
+                                             float scale, void* out, void* stream) {
+  MSPR_REQUIRE(batch >= 1 && n_heads >= 1 && n_rows >= 0 && win_rows >= 0, "sparse_mla_decode_static: bad size argument");
+  const size_t need = workspace_bytes(batch, n_heads, (int64_t)n_rows + win_rows);
+  MSPR_REQUIRE(need <= kStaticBytes,
+               "sparse_mla_decode_static: batch %d x %d heads x %d keys needs %zu bytes of scratch, the built-in "
+               "scratch holds %zu (at most 256 key ranges): use mspr_sparse_mla_decode with a workspace",
+               batch, n_heads, n_rows + win_rows, need, kStaticBytes);
+  void* ws = nullptr;
+  int rc = static_scratch(&ws);
+  if (rc != MSPR_OK) return rc;
+  return sparse_mla_decode_impl(q, kv, rows, sinks, dtype, batch, n_heads, k_dim, v_dim, n_pool, n_rows, row_mul,
+                                row_add, win_start, win_rows, scale, out, ws, kStaticBytes, stream);
 }
