@@ -222,24 +222,26 @@ size_t mspr_sdpa_decode_q8_workspace_bytes(int batch, int n_kv_heads, int64_t n_
 /* One-token GQA decode attention over an MLX affine 8-bit KV cache, dequantised in-kernel.
  * Replaces mlx_kquant.sdpa_decode_q8 as called from runtime/qwen/full_attention.py:323
  * (third-party Metal operator, not vendored; arguments follow that call site).
- * queries: f32 [batch,n_q_heads,1,256]; k_wq/v_wq: uint32 [batch,n_kv_heads,n_keys,64] (four codes
- * per word, lowest byte first); scales and biases: [batch,n_kv_heads,n_keys,4] of sb_dtype,
+ * queries: f32 [batch,n_q_heads,1,256]; k_wq/v_wq: uint32 [batch,n_kv_heads,kv_rows,64] (four codes
+ * per word, lowest byte first); scales and biases: [batch,n_kv_heads,kv_rows,4] of sb_dtype,
  * value = code*scale + bias per 64 elements; out: f32 [batch,n_q_heads,1,256].
+ * kv_rows >= n_keys is the row capacity of the cache buffers: the first n_keys rows of every head are
+ * attended, so a cache that grows in blocks is passed as it lies in memory, without a trimmed copy.
  * group_size must be 64 and bits 8; n_q_heads/n_kv_heads <= 16. */
 int mspr_sdpa_decode_q8(const void* queries, int q_dtype, const void* k_wq, const void* k_scales,
                         const void* k_biases, const void* v_wq, const void* v_scales,
                         const void* v_biases, int sb_dtype, int batch, int n_q_heads, int n_kv_heads,
-                        int head_dim, int64_t n_keys, float scale, int group_size, int bits, void* out,
-                        void* workspace, size_t workspace_bytes, void* stream);
+                        int head_dim, int64_t n_keys, int64_t kv_rows, float scale, int group_size, int bits,
+                        void* out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Extension (BASELINE config 3): the same decode over a Q8_0 cache — int8 codes
- * [batch,n_kv_heads,n_keys,256] with one float16 scale per 32 elements
- * [batch,n_kv_heads,n_keys,8], value = code*scale. queries/out: [batch,n_q_heads,256] of q_dtype
- * (f32|f16|bf16). */
+ * [batch,n_kv_heads,kv_rows,256] with one float16 scale per 32 elements
+ * [batch,n_kv_heads,kv_rows,8], value = code*scale (the first n_keys rows of every head are attended).
+ * queries/out: [batch,n_q_heads,256] of q_dtype (f32|f16|bf16). */
 int mspr_sdpa_decode_q8_0(const void* queries, int q_dtype, const void* k_codes, const void* k_scales,
                           const void* v_codes, const void* v_scales, int batch, int n_q_heads,
-                          int n_kv_heads, int head_dim, int64_t n_keys, float scale, void* out,
-                          void* workspace, size_t workspace_bytes, void* stream);
+                          int n_kv_heads, int head_dim, int64_t n_keys, int64_t kv_rows, float scale,
+                          void* out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Causal chunked-prefill GQA attention over a dense 16-bit KV cache that already holds the chunk:
  * query row i (position past_len + i) attends keys [0, past_len + i].
@@ -265,16 +267,20 @@ size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_q_heads, int n_k
  * Replaces mlx_kquant.sdpa_fa_prefill_q8 as called from runtime/qwen/full_attention.py:372
  * (third-party Metal operator, not vendored; arguments follow that call site and the helper at
  * tests/test_qwen_flash_prefill_attention.py:361-375).
- * queries/out: f32 [batch,n_q_heads,q_len,256]; pk_wq/pv_wq: uint32 [batch,n_kv_heads,past_len,64];
- * their scales and biases: [batch,n_kv_heads,past_len,4] of sb_dtype; self_k/self_v:
- * [batch,n_kv_heads,q_len,256] of self_dtype (already passed through the 8-bit round trip by the
- * caller). past_len may be 0 (the prefix pointers are then ignored). */
+ * queries/out: f32 [batch,n_q_heads,q_len,256]; pk_wq/pv_wq: uint32 [batch,n_kv_heads,past_rows,64];
+ * their scales and biases: [batch,n_kv_heads,past_rows,4] of sb_dtype, past_rows >= past_len being the
+ * row capacity of the prefix buffers (the first past_len rows of every head are the prefix);
+ * self_k/self_v: [batch,n_kv_heads,q_len,256] of self_dtype (already passed through the 8-bit round
+ * trip by the caller). past_len may be 0 (the prefix pointers are then ignored).
+ * The chunk's own rows, the last past_len % 32 prefix rows and the queries are staged as float16 MFMA
+ * operands whatever self_dtype is: chunk rows beyond +-65504 saturate there, queries beyond it become
+ * infinite, and everything keeps 11 significant bits. */
 int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, const void* pk_scales,
                             const void* pk_biases, const void* pv_wq, const void* pv_scales,
                             const void* pv_biases, int sb_dtype, const void* self_k, const void* self_v,
                             int self_dtype, int batch, int n_q_heads, int n_kv_heads, int head_dim,
-                            int q_len, int64_t past_len, float scale, int group_size, int bits, void* out,
-                            void* workspace, size_t workspace_bytes, void* stream);
+                            int q_len, int64_t past_len, int64_t past_rows, float scale, int group_size,
+                            int bits, void* out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------ measurement */
 

@@ -66,10 +66,10 @@ SIGNATURES = {
     "mspr_sdpa_decode_q8_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),
     "mspr_sdpa_decode_q8": (
         c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
+                c_int, c_int, c_int64, c_int64, c_float, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_sdpa_decode_q8_0": (
         c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int64,
-                c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
+                c_int64, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_flash_prefill": (
         c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_float,
                 c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -77,7 +77,7 @@ SIGNATURES = {
     "mspr_sdpa_fa_prefill_q8_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int64]),
     "mspr_sdpa_fa_prefill_q8": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p, c_void_p,
+                c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_int64, c_float, c_int, c_int, c_void_p, c_void_p,
                 c_size_t, c_void_p]),
     "mspr_profile_enable": (c_int, [c_int]),
     "mspr_profile_collect": (c_int, [c_int, c_void_p, c_int]),

@@ -47,8 +47,9 @@ struct PrefillArgs {
   // quantised-prefix form only: tiles [0, q8_tiles) come from the affine 8-bit prefix below, the rest
   // from k / v, which then hold float16 rows for keys [32 q8_tiles, past_len + q_len)
   int q8_tiles;
-  const void* pk_wq;  // [B, Hkv, past_len, 256] codes
-  const void* pk_s;   // [B, Hkv, past_len, 4]
+  int64_t past_rows;  // rows allocated per (batch, kv head) in the prefix tensors; >= past_len
+  const void* pk_wq;  // [B, Hkv, past_rows, 256] codes
+  const void* pk_s;   // [B, Hkv, past_rows, 4]
   const void* pk_b;
   const void* pv_wq;
   const void* pv_s;
@@ -386,7 +387,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
       constexpr int kRawBytes = 2 * kCodeBytes + 4 * 512;
       constexpr int kRawBase = 2 * kStageBytes;      // the unpacked stages use the lower 64 KB
       static_assert(kRawBase + 3 * kRawBytes <= kLdsBytes, "raw ring does not fit");
-      const int64_t row0 = ((int64_t)b * a.n_kv_heads + kvh) * past;
+      const int64_t row0 = ((int64_t)b * a.n_kv_heads + kvh) * a.past_rows;
       const uint8_t* kc = reinterpret_cast<const uint8_t*>(a.pk_wq) + row0 * kD;
       const uint8_t* vc = reinterpret_cast<const uint8_t*>(a.pv_wq) + row0 * kD;
       // scale / bias copies: wave w moves array w & 3 (K scale, K bias, V scale, V bias), 4 bytes per lane; with
@@ -533,7 +534,7 @@ __global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, con
   const int64_t key = (int64_t)a.q8_tiles * kTile + j;
   float kx, vx;
   if (key < a.past_len) {
-    const int64_t row = bh * a.past_len + key;
+    const int64_t row = bh * a.past_rows + key;
     const float ks = load_as_f32<SDT>(a.pk_s, row * 4 + d / 64), kb = load_as_f32<SDT>(a.pk_b, row * 4 + d / 64);
     const float vs = load_as_f32<SDT>(a.pv_s, row * 4 + d / 64), vb = load_as_f32<SDT>(a.pv_b, row * 4 + d / 64);
     kx = (float)reinterpret_cast<const uint8_t*>(a.pk_wq)[row * kD + d] * ks + kb;
@@ -551,6 +552,10 @@ __global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, con
       vx = load_as_f32<MSPR_BF16>(self_v, off);
     }
   }
+  // float16 staging: values beyond its range saturate instead of becoming infinite (an infinite key or value
+  // turns the whole output row into NaN)
+  kx = __builtin_amdgcn_fmed3f(kx, -65504.0f, 65504.0f);
+  vx = __builtin_amdgcn_fmed3f(vx, -65504.0f, 65504.0f);
   tail_k[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(kx);
   tail_v[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(vx);
 }
@@ -731,9 +736,10 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
                                        const void* pk_biases, const void* pv_wq, const void* pv_scales,
                                        const void* pv_biases, int sb_dtype, const void* self_k, const void* self_v,
                                        int self_dtype, int batch, int n_q_heads, int n_kv_heads, int head_dim,
-                                       int q_len, int64_t past_len, float scale, int group_size, int bits, void* out,
-                                       void* workspace, size_t workspace_bytes, void* stream) {
+                                       int q_len, int64_t past_len, int64_t past_rows, float scale, int group_size,
+                                       int bits, void* out, void* workspace, size_t workspace_bytes, void* stream) {
   MSPR_REQUIRE(group_size == 64 && bits == 8, "sdpa_fa_prefill_q8: only group_size=64, bits=8 is supported");
+  MSPR_REQUIRE(past_rows >= past_len, "sdpa_fa_prefill_q8: past_rows (rows allocated per head) must cover past_len");
   MSPR_REQUIRE(queries && self_k && self_v && out, "sdpa_fa_prefill_q8: null pointer");
   MSPR_REQUIRE(past_len == 0 || (pk_wq && pk_scales && pk_biases && pv_wq && pv_scales && pv_biases),
                "sdpa_fa_prefill_q8: null pointer");
@@ -774,6 +780,7 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
   a.rep_shift = rep == 1 ? 0 : rep == 2 ? 1 : rep == 4 ? 2 : 3;
   a.q_blocks = prefill_q_blocks(rep, q_len);
   a.q8_tiles = (int)(past_len / kTile);
+  a.past_rows = past_rows;
   a.n_splits = prefill_choose_splits(batch, n_kv_heads, a.q_blocks, past_len, q_len);
   if (a.n_splits > 1) {
     const size_t tail = ((size_t)batch * n_kv_heads * tail_rows * kRowBytes * 2 + 255) / 256 * 256;

@@ -40,6 +40,7 @@ struct Q8Args {
   const void* v_biases;
   int batch, n_q_heads, n_kv_heads;
   int64_t n_keys;
+  int64_t kv_rows;  // rows allocated per (batch, kv head); >= n_keys
   float scale_log2;
   int n_splits;
   int keys_per_split;
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(64 * kQ8Waves, 1) void q8_decode_split_kernel(Q8Arg
   int64_t k1 = k0 + a.keys_per_split;
   if (k1 > N) k1 = N;
 
-  const int64_t kv_row0 = ((int64_t)b * a.n_kv_heads + kvh) * N;  // first key row of this (b, kv head)
+  const int64_t kv_row0 = ((int64_t)b * a.n_kv_heads + kvh) * a.kv_rows;  // first key row of this (b, kv head)
   const uint8_t* kc = reinterpret_cast<const uint8_t*>(a.k_codes) + kv_row0 * kD;
   const uint8_t* vc = reinterpret_cast<const uint8_t*>(a.v_codes) + kv_row0 * kD;
   constexpr int kGroups = FMT == kFmtQ8_0 ? 8 : 4;  // scale groups per row
@@ -592,7 +593,9 @@ int q8_common_checks(const char* what, const void* q, const void* kc, const void
   return MSPR_OK;
 }
 
-void q8_fill_args(Q8Args& a, int batch, int n_q_heads, int n_kv_heads, int64_t n_keys, float scale, void* workspace) {
+void q8_fill_args(Q8Args& a, int batch, int n_q_heads, int n_kv_heads, int64_t n_keys, int64_t kv_rows, float scale,
+                  void* workspace) {
+  a.kv_rows = kv_rows;
   a.batch = batch;
   a.n_q_heads = n_q_heads;
   a.n_kv_heads = n_kv_heads;
@@ -616,9 +619,10 @@ extern "C" size_t mspr_sdpa_decode_q8_workspace_bytes(int batch, int n_kv_heads,
 extern "C" int mspr_sdpa_decode_q8(const void* queries, int q_dtype, const void* k_wq, const void* k_scales,
                                    const void* k_biases, const void* v_wq, const void* v_scales,
                                    const void* v_biases, int sb_dtype, int batch, int n_q_heads, int n_kv_heads,
-                                   int head_dim, int64_t n_keys, float scale, int group_size, int bits, void* out,
-                                   void* workspace, size_t workspace_bytes, void* stream) {
+                                   int head_dim, int64_t n_keys, int64_t kv_rows, float scale, int group_size,
+                                   int bits, void* out, void* workspace, size_t workspace_bytes, void* stream) {
   MSPR_REQUIRE(group_size == 64 && bits == 8, "sdpa_decode_q8: only group_size=64, bits=8 is supported");
+  MSPR_REQUIRE(kv_rows >= n_keys, "sdpa_decode_q8: kv_rows (rows allocated per head) must cover n_keys");
   MSPR_REQUIRE(q_dtype == MSPR_F32, "sdpa_decode_q8: queries must be float32");
   MSPR_REQUIRE(sb_dtype >= MSPR_F32 && sb_dtype <= MSPR_BF16, "sdpa_decode_q8: scales/biases must be f32, f16 or bf16");
   MSPR_REQUIRE(k_biases && v_biases, "sdpa_decode_q8: null pointer");
@@ -634,7 +638,7 @@ extern "C" int mspr_sdpa_decode_q8(const void* queries, int q_dtype, const void*
   a.v_scales = v_scales;
   a.v_biases = v_biases;
   a.out = out;
-  q8_fill_args(a, batch, n_q_heads, n_kv_heads, n_keys, scale, workspace);
+  q8_fill_args(a, batch, n_q_heads, n_kv_heads, n_keys, kv_rows, scale, workspace);
   hipStream_t st = (hipStream_t)stream;
   if (sb_dtype == MSPR_F32) return q8_launch<kFmtAffine, MSPR_F32, MSPR_F32>(a, st);
   if (sb_dtype == MSPR_F16) return q8_launch<kFmtAffine, MSPR_F32, MSPR_F16>(a, st);
@@ -643,8 +647,9 @@ extern "C" int mspr_sdpa_decode_q8(const void* queries, int q_dtype, const void*
 
 extern "C" int mspr_sdpa_decode_q8_0(const void* queries, int q_dtype, const void* k_codes, const void* k_scales,
                                      const void* v_codes, const void* v_scales, int batch, int n_q_heads,
-                                     int n_kv_heads, int head_dim, int64_t n_keys, float scale, void* out,
-                                     void* workspace, size_t workspace_bytes, void* stream) {
+                                     int n_kv_heads, int head_dim, int64_t n_keys, int64_t kv_rows, float scale,
+                                     void* out, void* workspace, size_t workspace_bytes, void* stream) {
+  MSPR_REQUIRE(kv_rows >= n_keys, "sdpa_decode_q8_0: kv_rows (rows allocated per head) must cover n_keys");
   MSPR_REQUIRE(q_dtype >= MSPR_F32 && q_dtype <= MSPR_BF16, "sdpa_decode_q8_0: queries must be f32, f16 or bf16");
   int rc = q8_common_checks("sdpa_decode_q8_0", queries, k_codes, k_scales, v_codes, v_scales, out, batch, n_q_heads,
                             n_kv_heads, head_dim, n_keys, workspace, workspace_bytes);
@@ -656,7 +661,7 @@ extern "C" int mspr_sdpa_decode_q8_0(const void* queries, int q_dtype, const voi
   a.v_codes = v_codes;
   a.v_scales = v_scales;
   a.out = out;
-  q8_fill_args(a, batch, n_q_heads, n_kv_heads, n_keys, scale, workspace);
+  q8_fill_args(a, batch, n_q_heads, n_kv_heads, n_keys, kv_rows, scale, workspace);
   hipStream_t st = (hipStream_t)stream;
   if (q_dtype == MSPR_F32) return q8_launch<kFmtQ8_0, MSPR_F32, MSPR_F16>(a, st);
   if (q_dtype == MSPR_F16) return q8_launch<kFmtQ8_0, MSPR_F16, MSPR_F16>(a, st);

@@ -67,18 +67,14 @@ def _indexer_q_qat_v2_enabled() -> bool:
 
 def indexed_mixed_attention_decode(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
                                    ratio: int = 4, raw_start: int = 0):
-    """One-token DS4 indexed mixed attention (reference :1496).
+    """Decode consumer of the indexed mixed attention: one query token (reference :1496).
 
-    Args:
-        q: float32 ``[n_heads, 512]`` query heads (rounded to half on load).
-        raw_kv: float16 ``[raw_cap, 512]`` contiguous/circular raw KV rows.
-        comp_kv: float16 ``[n_comp, 512]`` compressed KV rows.
-        topk: int32 ``[top_k]`` selected compressed row ids (other integer
-            dtypes are cast, as in the reference).
-        sinks: float32 ``[n_heads]`` attention sink logits (cast if needed).
-
-    Returns:
-        float32 ``[n_heads, 512]``.
+    Operands: ``q`` is ``[n_heads, 512]`` float32 and is rounded to half precision when loaded;
+    ``raw_kv`` ``[raw_cap, 512]`` float16 is the sliding-window ring, whose oldest row sits at
+    ``raw_start``; ``comp_kv`` ``[n_comp, 512]`` float16 is the compressed pool; ``topk`` ``[top_k]``
+    names the pool rows to visit (any integer type, converted to int32 as the reference does);
+    ``sinks`` ``[n_heads]`` holds one sink logit per head (converted to float32 if needed).
+    The result is float32 ``[n_heads, 512]``.
     """
     if q.ndim != 2 or raw_kv.ndim != 2 or comp_kv.ndim != 2:
         raise ValueError("q, raw_kv, and comp_kv must be rank-2")
@@ -206,18 +202,14 @@ def _run_prefill(q, raw_kv, comp_kv, topk, sinks, *, batch, n_heads, n_tokens, s
 
 def indexed_mixed_attention_prefill(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
                                     ratio: int = 4, raw_start: int = 0):
-    """Batch-token indexed mixed attention, DS4-c layout (reference :2030).
+    """Prefill consumer on token-major operands: the decode rules applied to every token of a chunk
+    (reference :2030).
 
-    Args:
-        q: float32 ``[tokens, n_heads, 512]`` query heads.
-        raw_kv: float16 ``[raw_cap, 512]`` local raw KV rows; the newest row holds position
-            ``pos0 + tokens - 1``.
-        comp_kv: float16 ``[n_comp, 512]`` compressed KV rows.
-        topk: int32 ``[tokens, top_k]`` selected compressed row ids.
-        sinks: float32 ``[n_heads]`` attention sink logits.
-
-    Returns:
-        float32 ``[tokens, n_heads, 512]``.
+    Token ``t`` sits at position ``pos0 + t``. ``q`` is ``[tokens, n_heads, 512]`` float32; the ring
+    ``raw_kv`` ``[raw_cap, 512]`` float16 ends with the row of the chunk's last token (position
+    ``pos0 + tokens - 1``); ``comp_kv`` ``[n_comp, 512]`` float16 is the compressed pool; row ``t`` of
+    ``topk`` ``[tokens, top_k]`` lists the pool rows of token ``t``; ``sinks`` ``[n_heads]`` are the
+    per-head sink logits. The result is float32 with the shape of ``q``.
     """
     if q.ndim != 3 or raw_kv.ndim != 2 or comp_kv.ndim != 2:
         raise ValueError("q must be rank-3 and raw_kv/comp_kv rank-2")
@@ -313,15 +305,11 @@ def _launch_live(q, raw_kv, comp_kv, topk, sinks, dims, *, pos0, window, ratio, 
 
 def indexed_mixed_attention_prefill_live_f16(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
                                              ratio: int = 4, raw_start: int = 0):
-    """Indexed prefill attention on the live BHLD layout, float16 queries (reference :1571).
+    """The prefill consumer on the layouts the attention block holds, half-precision queries (reference :1571).
 
-    Args:
-        q: float16 ``[batch, n_heads, tokens, 512]``.
-        raw_kv: float16 ``[batch, 1, raw_cap, 512]``; comp_kv: float16 ``[batch, n_comp, 512]``.
-        topk: int32 ``[batch, tokens, top_k]``; sinks: float32 ``[n_heads]``.
-
-    Returns:
-        float32 ``[batch, n_heads, tokens, 512]``.
+    ``q`` is head-major ``[batch, n_heads, tokens, 512]`` float16, the ring ``[batch, 1, raw_cap, 512]``
+    and the pool ``[batch, n_comp, 512]`` float16, ``topk`` ``[batch, tokens, top_k]`` int32 and ``sinks``
+    ``[n_heads]`` float32; the float32 result has the shape of ``q``.
     """
     dims = _validate_live(q, raw_kv, comp_kv, topk, sinks, torch.float16,
                           "live prefill probe requires q to be float16", raw_start)
@@ -446,3 +434,60 @@ def indexer_q_qat_live(q):
                                             _lib.stream_ptr())
     _lib.check(rc, "indexer_q_qat_live")
     return out
+
+
+def _composed_sink_attention(qh, rows, sinks_h):
+    """softmax(q . rows^T / sqrt(D), with one sink logit per head in the denominator) . rows, float32:
+    the composition that ``scaled_dot_product_attention(..., sinks=)`` computes in the reference forms."""
+    head_dim = int(qh.shape[-1])
+    if int(rows.shape[0]) == 0:
+        return torch.zeros(qh.shape, dtype=torch.float32, device=qh.device)
+    logits = (qh.float() @ rows.float().T) * (float(head_dim) ** -0.5)
+    full = torch.cat([logits, sinks_h.float()[:, None]], dim=1)
+    prob = torch.softmax(full, dim=1)[:, :-1]
+    return prob @ rows.float()
+
+
+def mlx_selected_rows_attention_reference(q, raw_kv, comp_kv, topk, sinks):
+    """Composed selected-row consumer kept as correctness and speed reference (reference :2111).
+
+    Every ring row, then ``comp_kv[topk]``, attended by float16 ``q`` with float16 sinks; no visibility
+    rules. Built from tensor operations on the device (the reference composes MLX operations the same
+    way): it is the form the kernels are compared with, not a kernel path. The name is the reference's.
+    """
+    selected = torch.index_select(comp_kv, 0, topk.to(torch.int64))
+    full = torch.cat([raw_kv, selected], dim=0)
+    return _composed_sink_attention(q.to(torch.float16), full, sinks.to(torch.float16)).reshape(q.shape)
+
+
+def mlx_indexed_mixed_attention_prefill_reference(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
+                                                  ratio: int = 4):
+    """Composed per-token reference of the prefill consumer (reference :2133).
+
+    Token ``t`` attends the ring rows of positions ``[max(first_raw, pos0+t+1-window), pos0+t]`` (ring
+    starting at row 0) and the pool rows whose ids lie in ``[0, (pos0+t+1)//ratio)`` — ids outside that
+    range are dropped wherever they stand, where the kernel stops at the first one. q ``[tokens,
+    n_heads, 512]``; result float32 of the same shape.
+    """
+    n_tokens, n_heads, head_dim = (int(v) for v in q.shape)
+    n_raw = int(raw_kv.shape[0])
+    raw_last_pos = int(pos0) + n_tokens - 1
+    first_raw_pos = raw_last_pos + 1 - n_raw
+    sinks_h = sinks.to(torch.float16)
+    rows_out = []
+    for token in range(n_tokens):
+        qpos = int(pos0) + token
+        window_first = qpos + 1 - int(window) if window and qpos + 1 > window else 0
+        first = max(first_raw_pos, window_first)
+        last = min(qpos, raw_last_pos)
+        parts = []
+        if first <= last:
+            parts.append(raw_kv[first - first_raw_pos:last - first_raw_pos + 1])
+        visible = min((qpos + 1) // int(ratio), int(comp_kv.shape[0]))
+        ids = topk[token].to(torch.int64)
+        ids = ids[(ids >= 0) & (ids < visible)]
+        if int(ids.numel()):
+            parts.append(torch.index_select(comp_kv, 0, ids))
+        full = torch.cat(parts, dim=0) if parts else raw_kv[:0]
+        rows_out.append(_composed_sink_attention(q[token].to(torch.float16), full, sinks_h))
+    return torch.stack(rows_out, dim=0)

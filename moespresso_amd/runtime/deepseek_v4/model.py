@@ -42,19 +42,29 @@ class DeepseekV4RuntimeLoadError(RuntimeError):
 
 # ---------------------------------------------------------------- row transforms
 
-def _dsv4_indexer_qat(x: torch.Tensor) -> torch.Tensor:
+def _rows_argument(args, name: str) -> torch.Tensor:
+    """The reference's row helpers take its array-library module as a leading positional (``f(mx, x)``);
+    both ``f(x)`` and ``f(module, x)`` are accepted here and the module handle is ignored."""
+    if len(args) == 1:
+        return args[0]
+    if len(args) == 2 and not isinstance(args[0], torch.Tensor):
+        return args[1]
+    raise TypeError(f"{name} takes the rows, optionally behind an array-module handle")
+
+
+def _dsv4_indexer_qat(*args) -> torch.Tensor:
     """Hadamard-128 + e2m1 activation round trip of 128-wide rows, float32 out (reference :745)."""
-    return indexer_score_kernel.indexer_qat_rows(x)
+    return indexer_score_kernel.indexer_qat_rows(_rows_argument(args, "_dsv4_indexer_qat"))
 
 
-def _dsv4_decode_indexer_qat(x: torch.Tensor):
+def _dsv4_decode_indexer_qat(*args):
     """Decode-side QAT; returns ``(rows, used_kernel)`` (reference :772).
 
     There is one implementation here, the kernel; the kill switch of the reference selects its composed
     chain, which computes the same bits, so it only changes the engagement flag.
     """
     used = os.environ.get(_DSV4_DECODE_QAT_KERNEL_ENV, "1") != "0"
-    return indexer_score_kernel.indexer_qat_rows(x), used
+    return indexer_score_kernel.indexer_qat_rows(_rows_argument(args, "_dsv4_decode_indexer_qat")), used
 
 
 def _deepseek_v4_fp8_kv_roundtrip(x: torch.Tensor, *, head_dim: int = 512, rot_dim: int = 64) -> torch.Tensor:
@@ -182,9 +192,24 @@ class _IndexerDS4ScoreContract:
         key = f"_moespresso_dsv4_indexer_score_contract_{name}"
         setattr(self, key, getattr(self, key) + int(amount))
 
-    def __call__(self, x, q_residual, rope, position_rope, cache, start_pos):
+    def _engages(self, x) -> bool:
+        """Everything that decides whether this call is served here, checked before any cache state moves:
+        the decode shape, the score-kernel gate and the indexer geometry the kernel serves."""
         B, L, _ = x.shape
         if int(B) != 1 or int(L) != 1:
+            return False
+        if not indexer_score_kernel._ENABLED or not indexer_score_kernel._metal_available():
+            return False
+        ind = self._original
+        if int(ind.head_dim) != 128 or not 1 <= int(ind.n_heads) <= 64:
+            return False
+        return x.dtype in (torch.float32, torch.float16, torch.bfloat16)
+
+    def __call__(self, x, q_residual, rope, position_rope, cache, start_pos):
+        # The wrapped indexer advances the stateful compressor itself, so it may only be entered while
+        # this call has not: the decision is taken up front, and once the compressor has run the call is
+        # finished here whatever the operands look like (the reference finishes inline as well, :1040-1056).
+        if not self._engages(x):
             return self._original(x, q_residual, rope, position_rope, cache, start_pos)
         ind = self._original
         pooled = ind.compressor(x, rope, cache, start_pos, state_key="indexer_state")
@@ -206,13 +231,12 @@ class _IndexerDS4ScoreContract:
         self._bump("cached_pooled_rows", cached_rows)
         self._bump("new_qat_pooled_rows", new_rows)
         weights = ind.weights_proj(x).to(torch.float32) * (heads ** -0.5)
-        if indexer_score_kernel.fused_qat_scores_eligible(q, pooled_qat, weights):
-            scores = indexer_score_kernel.fused_qat_indexer_scores(q, pooled_qat, weights, float(ind.scale))
-            self._bump("fused_score_calls", 1)
-            scores = scores.reshape(1, 1, pooled_rows)
-        else:
-            return self._original(x, q_residual, rope, position_rope, cache, start_pos)
-        return indexer_score_kernel.topk_select(scores, topk_rows)
+        if q.dtype not in (torch.float32, torch.float16, torch.bfloat16):
+            q = q.to(torch.float32)
+        scores = indexer_score_kernel.fused_qat_indexer_scores(
+            q, pooled_qat.to(torch.float32), weights.reshape(1, 1, heads), float(ind.scale))
+        self._bump("fused_score_calls", 1)
+        return indexer_score_kernel.topk_select(scores.reshape(1, 1, pooled_rows), topk_rows)
 
 
 # ---------------------------------------------------------------- fused ratio-4 decode attention
@@ -403,9 +427,9 @@ def _patch_deepseek_v4_ratio4_decode_fused_attention(model, *, cache_cls) -> int
 
 # ---------------------------------------------------------------- ratio-4 prefill fast path
 
-def _dsv4_prefill_pooled_qat(x: torch.Tensor) -> torch.Tensor:
+def _dsv4_prefill_pooled_qat(*args) -> torch.Tensor:
     """QAT of pooled indexer rows on the prefill path (reference :752); same kernel as the decode side."""
-    return indexer_score_kernel.indexer_qat_rows(x)
+    return indexer_score_kernel.indexer_qat_rows(_rows_argument(args, "_dsv4_prefill_pooled_qat"))
 
 
 class _Ratio4PrefillFastAttention:

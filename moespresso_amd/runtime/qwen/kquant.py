@@ -44,6 +44,30 @@ def _check_q8_triplet(name, wq, scales, biases, batch, n_keys=None):
         raise ValueError("keys and values disagree on the number of cached tokens")
 
 
+def _row_capacity(t, n_rows: int):
+    """Row capacity of a ``[B, H, n_rows, W]`` tensor that is the first ``n_rows`` rows of every head of a
+    dense ``[B, H, capacity, W]`` buffer (what a cache that grows in blocks hands out), else ``None``."""
+    B, H, N, W = (int(v) for v in t.shape)
+    sb, sh, sn, sw = (int(v) for v in t.stride())
+    if sw != 1 or sn != W:
+        return None
+    if B * H == 1:
+        return N
+    cap = (sh if H > 1 else sb) // W if W else 0
+    if cap < N or (H > 1 and sh != cap * W) or (B > 1 and sb != H * cap * W):
+        return None
+    return cap
+
+
+def _cache_operands(tensors, n_rows: int):
+    """The cache tensors as the library reads them: untouched when all of them are leading-row views of dense
+    buffers with one common row capacity (no copy), otherwise dense copies with capacity ``n_rows``."""
+    caps = [_row_capacity(t, n_rows) for t in tensors]
+    if caps[0] is not None and all(c == caps[0] for c in caps):
+        return list(tensors), caps[0]
+    return [t.contiguous() for t in tensors], n_rows
+
+
 def quantize(x, group_size: int = 64, bits: int = 8):
     """Affine 8-bit quantisation over the last axis (the role of ``mx.quantize`` on the cache write path).
 
@@ -186,14 +210,14 @@ def sdpa_decode_q8(queries, k_wq, k_scales, k_biases, v_wq, v_scales, v_biases, 
     if N < 1:
         raise ValueError("the cache must hold at least one token")
     _lib.require_device(queries, k_wq, k_scales, k_biases, v_wq, v_scales, v_biases)
-    tensors = [t.contiguous() for t in (queries, k_wq, k_scales, k_biases, v_wq, v_scales, v_biases)]
-    q, kw, ks, kb, vw, vs, vb = tensors
+    q = queries.contiguous()
+    (kw, ks, kb, vw, vs, vb), kv_rows = _cache_operands((k_wq, k_scales, k_biases, v_wq, v_scales, v_biases), N)
     out = torch.empty_like(q)
     if workspace is None:
         workspace = _lib.q8_decode_workspace(B, Hkv, N, q.device)
     _lib.check(_lib.lib().mspr_sdpa_decode_q8(
         _lib.ptr(q), _lib.DTYPE_CODE[q.dtype], _lib.ptr(kw), _lib.ptr(ks), _lib.ptr(kb), _lib.ptr(vw), _lib.ptr(vs),
-        _lib.ptr(vb), _lib.DTYPE_CODE[ks.dtype], B, Hq, Hkv, _HEAD_DIM, N, float(scale), 64, 8, _lib.ptr(out),
+        _lib.ptr(vb), _lib.DTYPE_CODE[ks.dtype], B, Hq, Hkv, _HEAD_DIM, N, kv_rows, float(scale), 64, 8, _lib.ptr(out),
         _lib.ptr(workspace), workspace.numel() * workspace.element_size(), _lib.stream_ptr()), "sdpa_decode_q8")
     return out
 
@@ -228,13 +252,14 @@ def sdpa_decode_q8_0(queries, k_codes, k_scales, v_codes, v_scales, scale, *, wo
     if N < 1:
         raise ValueError("the cache must hold at least one token")
     _lib.require_device(queries, k_codes, k_scales, v_codes, v_scales)
-    q, kc, ks, vc, vs = [t.contiguous() for t in (queries, k_codes, k_scales, v_codes, v_scales)]
+    q = queries.contiguous()
+    (kc, ks, vc, vs), kv_rows = _cache_operands((k_codes, k_scales, v_codes, v_scales), N)
     out = torch.empty_like(q)
     if workspace is None:
         workspace = _lib.q8_decode_workspace(B, Hkv, N, q.device)
     _lib.check(_lib.lib().mspr_sdpa_decode_q8_0(
         _lib.ptr(q), _lib.DTYPE_CODE[q.dtype], _lib.ptr(kc), _lib.ptr(ks), _lib.ptr(vc), _lib.ptr(vs), B, Hq, Hkv,
-        _HEAD_DIM, N, float(scale), _lib.ptr(out), _lib.ptr(workspace),
+        _HEAD_DIM, N, kv_rows, float(scale), _lib.ptr(out), _lib.ptr(workspace),
         workspace.numel() * workspace.element_size(), _lib.stream_ptr()), "sdpa_decode_q8_0")
     return out
 
@@ -276,8 +301,9 @@ def sdpa_fa_prefill_q8(queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, p
     if L < 1:
         raise ValueError("the chunk must hold at least one token")
     _lib.require_device(queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, pv_biases, self_k, self_v)
-    q, kw, ks, kb, vw, vs, vb, sk, sv = [
-        t.contiguous() for t in (queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, pv_biases, self_k, self_v)]
+    q, sk, sv = queries.contiguous(), self_k.contiguous(), self_v.contiguous()
+    (kw, ks, kb, vw, vs, vb), past_rows = _cache_operands(
+        (pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, pv_biases), P)
     out = torch.empty_like(q)
     if workspace is None:
         nbytes = int(_lib.lib().mspr_sdpa_fa_prefill_q8_workspace_bytes(B, Hq, Hkv, L, P))
@@ -285,7 +311,7 @@ def sdpa_fa_prefill_q8(queries, pk_wq, pk_scales, pk_biases, pv_wq, pv_scales, p
     _lib.check(_lib.lib().mspr_sdpa_fa_prefill_q8(
         _lib.ptr(q), _lib.ptr(kw), _lib.ptr(ks), _lib.ptr(kb), _lib.ptr(vw), _lib.ptr(vs), _lib.ptr(vb),
         _lib.DTYPE_CODE[ks.dtype], _lib.ptr(sk), _lib.ptr(sv), _lib.DTYPE_CODE[sk.dtype], B, Hq, Hkv, _HEAD_DIM, L, P,
-        float(scale), 64, 8, _lib.ptr(out), _lib.ptr(workspace), workspace.numel() * workspace.element_size(),
+        past_rows, float(scale), 64, 8, _lib.ptr(out), _lib.ptr(workspace), workspace.numel() * workspace.element_size(),
         _lib.stream_ptr()), "sdpa_fa_prefill_q8")
     return out
 

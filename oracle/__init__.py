@@ -26,6 +26,11 @@ would fail; "unpinned" = only self-consistency is available):
   rope / yarn                        pinned  (reference pinned inv-freq and angle values)
   sink attention / visit rules       pinned  (single-key+sink KAT, torch.softmax when sink=-inf,
                                      visibility KATs, brute-force row lists)
+  prefill visit rules / last_pos     pinned  (independent per-position walk with torch.softmax float64; the
+                                     composed reference form with its filter rule on sorted and unsorted ids)
+  fused_decode_prep                  pinned  (all-tie -> arange KAT, integer data against a brute-force
+                                     float64 sum and lexsort, prepared row against rope and FP8 parts)
+  round_bf16 / round_f16             pinned  (torch.bfloat16 / float16 casts incl. ties, inf, NaN, denormals)
   q8 quantisers (affine g64)         parity unpinned (MLX mx.quantize edge rules not in the
                                      reference tree; own documented rule, round trip bounded)
   gqa decode / causal flash prefill  pinned  (float64 torch.softmax closed form)

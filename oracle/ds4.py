@@ -722,6 +722,43 @@ def indexed_mixed_attention_prefill(q, raw_kv, comp_kv, topk, sinks, *, pos0: in
     return out
 
 
+def indexed_mixed_attention_prefill_reference(q, raw_kv, comp_kv, topk, sinks, *, pos0: int, window: int = 128,
+                                              ratio: int = 4) -> np.ndarray:
+    """The reference's composed per-token form (indexed_attention_kernel.py:2133-2180).
+
+    Differs from the kernel restated above in three ways: the ring starts at row 0 (no ``raw_start``), ids
+    outside ``[0, visible)`` are FILTERED OUT anywhere in the list (the kernel stops at the first id
+    ``>= visible``), and q and the sinks pass through float16. On ascending id lists, which is what the
+    prefill consumer is given (model.py:1451), filter and stop select the same rows.
+    q ``[T,H,512]``, raw_kv ``[n_raw,512]``, topk ``[T,k]`` -> float64 ``[T,H,512]``.
+    """
+    q = np.asarray(q)
+    n_tokens, _, head_dim = q.shape
+    raw = np.asarray(raw_kv).astype(F32)
+    comp = np.asarray(comp_kv).astype(F32)
+    n_raw = raw.shape[0]
+    raw_last_pos = int(pos0) + n_tokens - 1
+    first_raw_pos = raw_last_pos + 1 - n_raw
+    sinks_h = round_f16(np.asarray(sinks, dtype=F32))
+    out = np.zeros(q.shape, dtype=np.float64)
+    for t in range(n_tokens):
+        qpos = int(pos0) + t
+        window_first = qpos + 1 - int(window) if window and qpos + 1 > window else 0
+        first = max(first_raw_pos, window_first)
+        last = min(qpos, raw_last_pos)
+        parts = []
+        if first <= last:
+            parts.append(raw[first - first_raw_pos:last - first_raw_pos + 1])
+        visible = min((qpos + 1) // int(ratio), comp.shape[0])
+        ids = np.asarray(topk)[t].astype(np.int64)
+        ids = ids[(ids >= 0) & (ids < visible)]
+        if ids.size:
+            parts.append(comp[ids])
+        rows = np.concatenate(parts, axis=0) if parts else np.zeros((0, head_dim), dtype=F32)
+        out[t] = attend_rows_f64(round_f16(q[t].astype(F32)), rows, sinks_h, float(head_dim) ** -0.5)
+    return out
+
+
 # --------------------------------------------------------------------------
 # a6/a9: fused decode island
 # --------------------------------------------------------------------------

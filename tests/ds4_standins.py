@@ -67,14 +67,20 @@ class OtherCache(_CacheBase):
 
 
 class Compressor:
-    """Returns the pool held in the cache state (the steady-state token appends no pool row)."""
+    """Returns the pool held in the cache state (the steady-state token appends no pool row) and, like the
+    real one, keeps state per token: every call is recorded with its position and counted in the cache
+    state, so a token that advances it twice shows."""
 
     def __init__(self):
         self.calls = []
+        self.positions = []
 
     def __call__(self, x, rope, cache, offset, state_key="compressor_state"):
         self.calls.append(state_key)
-        return getattr(cache, state_key)["pooled"]
+        self.positions.append(int(offset))
+        state = getattr(cache, state_key)
+        state["advances"] = state.get("advances", 0) + 1
+        return state["pooled"]
 
 
 class Indexer:
@@ -86,8 +92,10 @@ class Indexer:
         self.weights_proj = _linear(hidden, n_heads, device, gen)
         self.stock_calls = 0
 
-    def __call__(self, *args):
+    def __call__(self, x, q_residual, rope, position_rope, cache, start_pos):
+        # the stock indexer advances its compressor itself
         self.stock_calls += 1
+        self.compressor(x, rope, cache, start_pos, state_key="indexer_state")
         return None
 
 

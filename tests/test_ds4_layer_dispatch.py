@@ -65,6 +65,82 @@ def test_every_contract_miss_delegates_before_touching_the_cache(monkeypatch):
     assert not wrapper._decode_eligible(x, good)
 
 
+def test_score_contract_decides_before_the_compressor_moves(monkeypatch):
+    # A decode token the contract does not serve (gate off, no device, geometry) must reach the wrapped
+    # indexer with the compressor untouched: the wrapped indexer advances it itself, and a second advance
+    # for the same token corrupts the pool (reference model.py:870-1056 never re-enters).
+    from moespresso_amd.runtime.deepseek_v4 import indexer_score_kernel as isk
+
+    attn = Attention("cpu", index_heads=64, topk=16)
+    contract = dsm._IndexerDS4ScoreContract(attn.indexer, 4, layer_index=0)
+    cache = steady_cache("cpu", rows=40)
+    x = torch.zeros((1, 1, 256), dtype=torch.float16)
+    q_res = torch.zeros((1, 1, 64), dtype=torch.float16)
+    monkeypatch.setattr(isk, "_ENABLED", False)
+    assert contract(x, q_res, None, None, cache, 100) is None
+    monkeypatch.setattr(isk, "_ENABLED", True)
+    monkeypatch.setattr(isk, "_metal_available", lambda: False)
+    assert contract(x, q_res, None, None, cache, 101) is None
+    monkeypatch.setattr(isk, "_metal_available", lambda: True)
+    attn.indexer.head_dim = 64                                   # geometry the score kernel does not serve
+    assert contract(x, q_res, None, None, cache, 102) is None
+    attn.indexer.head_dim = 128
+    assert contract(torch.zeros((1, 3, 256), dtype=torch.float16), q_res, None, None, cache, 103) is None
+    assert attn.indexer.stock_calls == 4
+    # one advance per token, all of them the wrapped indexer's own
+    assert attn.indexer.compressor.positions == [100, 101, 102, 103] and cache.indexer_state["advances"] == 4
+    c = "_moespresso_dsv4_indexer_score_contract_"
+    assert getattr(contract, c + "calls") == 0
+
+
+def test_score_tail_gates(monkeypatch):
+    # reference indexer_score_kernel.py:499-560: two env kill switches read per call, then shape and type
+    from moespresso_amd.runtime.deepseek_v4 import indexer_score_kernel as isk
+
+    monkeypatch.setattr(isk, "_metal_available", lambda: True)
+    assert isk.score_tail_enabled()
+    for env in ("MOESPRESSO_DSV4_INDEXER_CHAIN_TRIMS", "MOESPRESSO_DSV4_INDEXER_SCORE_TAIL"):
+        monkeypatch.setenv(env, "0")
+        assert not isk.score_tail_enabled()
+        monkeypatch.setenv(env, "1")
+        assert isk.score_tail_enabled()
+        monkeypatch.delenv(env)
+    scores = torch.zeros((1, 64, 1, 96))
+    w = torch.zeros((1, 1, 64), dtype=torch.bfloat16)
+    params = torch.tensor([7, 50], dtype=torch.int32)
+    assert isk.score_tail_eligible(scores, w, params)
+    assert isk.score_tail_eligible(torch.zeros((1, 32, 1, 1)), torch.zeros((1, 1, 32)), params)
+    assert not isk.score_tail_eligible(torch.zeros((1, 31, 1, 96)), torch.zeros((1, 1, 31)), params)   # < 32 heads
+    assert not isk.score_tail_eligible(torch.zeros((1, 65, 1, 96)), torch.zeros((1, 1, 65)), params)   # > 64 heads
+    assert not isk.score_tail_eligible(torch.zeros((2, 64, 1, 96)), w, params)                          # batch
+    assert not isk.score_tail_eligible(torch.zeros((1, 64, 2, 96)), w, params)                          # tokens
+    assert not isk.score_tail_eligible(torch.zeros((1, 64, 1, 0)), w, params)                           # empty
+    assert not isk.score_tail_eligible(scores.half(), w, params)                                        # score type
+    assert not isk.score_tail_eligible(scores, torch.zeros((1, 64)), params)                            # weight rank
+    assert not isk.score_tail_eligible(scores, torch.zeros((1, 1, 63)), params)                         # weight shape
+    assert not isk.score_tail_eligible(scores, w.double(), params)                                      # weight type
+    assert not isk.score_tail_eligible(scores, w, params.long())                                        # params type
+    assert not isk.score_tail_eligible(scores, w, params[:1])                                           # params size
+    monkeypatch.setattr(isk, "_metal_available", lambda: False)
+    assert not isk.score_tail_enabled() and not isk.score_tail_eligible(scores, w, params)
+
+
+def test_row_helpers_accept_the_reference_module_handle(monkeypatch):
+    # reference model.py:745,752,772 are called as f(mx, x)
+    from moespresso_amd.runtime.deepseek_v4 import indexer_score_kernel as isk
+
+    seen = []
+    monkeypatch.setattr(isk, "indexer_qat_rows", lambda rows: seen.append(rows) or rows)
+    x = torch.zeros((2, 128))
+    assert dsm._dsv4_indexer_qat(x) is x and dsm._dsv4_indexer_qat(torch, x) is x
+    assert dsm._dsv4_prefill_pooled_qat(torch, x) is x
+    rows, used = dsm._dsv4_decode_indexer_qat(torch, x)
+    assert rows is x and used and len(seen) == 4
+    import pytest
+    with pytest.raises(TypeError):
+        dsm._dsv4_indexer_qat(x, x)
+
+
 def test_cache_wrappers_are_idempotent_and_keep_the_originals():
     cache = steady_cache("cpu", rows=4)
     original = cache.update_and_fetch

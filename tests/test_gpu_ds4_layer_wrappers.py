@@ -231,12 +231,25 @@ def test_decode_score_contract_selects_on_the_fused_score_row(monkeypatch):
     # second token: the pool rows are reused
     contract(x, q_res, attn.compress_rope, attn.rope, cache, OFFSET + 1)
     assert getattr(contract, c + "cached_pooled_rows") == 200 and getattr(contract, c + "new_qat_pooled_rows") == 200
-    # prefill shapes go to the wrapped indexer, and so does a decode token while the score gate is off
+    # every token so far advanced the stateful compressor exactly once
+    assert attn.indexer.compressor.positions == [OFFSET, OFFSET + 1] and cache.indexer_state["advances"] == 2
+    # prefill shapes go to the wrapped indexer, and so does a decode token while the score gate is off:
+    # both before the compressor is touched, so the wrapped indexer's own advance is the only one
     contract(torch.zeros((1, 4, 256), dtype=torch.float16, device=DEV), q_res, None, None, cache, 0)
-    assert attn.indexer.stock_calls == 1
+    assert attn.indexer.stock_calls == 1 and cache.indexer_state["advances"] == 3
     monkeypatch.setattr(isk, "_ENABLED", False)
     assert contract(x, q_res, attn.compress_rope, attn.rope, cache, OFFSET + 2) is None
     assert attn.indexer.stock_calls == 2
+    assert attn.indexer.compressor.positions == [OFFSET, OFFSET + 1, 0, OFFSET + 2]
+    assert cache.indexer_state["advances"] == 4      # one advance per token, gate on or off
+    fused_before = getattr(contract, c + "fused_score_calls")
+    # once engaged the call finishes here even when the pool rows arrive in another float type
+    monkeypatch.setattr(isk, "_ENABLED", True)
+    cache.indexer_state.pop("pooled_qat"), cache.indexer_state.pop("pooled_qat_rows")
+    monkeypatch.setattr(dsm, "_dsv4_indexer_qat", lambda rows: isk.indexer_qat_rows(rows).to(torch.float16))
+    again = contract(x, q_res, attn.compress_rope, attn.rope, cache, OFFSET + 3)
+    assert tuple(again.shape) == (1, 1, 16) and attn.indexer.stock_calls == 2
+    assert getattr(contract, c + "fused_score_calls") == fused_before + 1 and cache.indexer_state["advances"] == 5
 
 
 def _prefill_setup(tokens, rows, *, topk, q_dtype=torch.float16):

@@ -181,3 +181,26 @@ def test_sdpa_fa_prefill_q8_full_size_sampled_rows():
         err = np.abs(got[:, :, row:row + 1] - want).max()
         assert err < 1e-2, (row, err)
 
+
+
+def test_sdpa_fa_prefill_q8_chunk_values_beyond_float16_range_saturate():
+    """The chunk's own K/V rows are staged as float16: values beyond +-65504 saturate there instead of turning
+    into inf (which would make every output row that attends them NaN). Rows inside the range are unaffected."""
+    from moespresso_amd.runtime.qwen import kquant
+
+    dev = _dev()
+    g = torch.Generator().manual_seed(9)
+    L = 40
+    q = torch.randn((1, 16, L, 256), generator=g) * 0.1
+    sk = torch.randn((1, 2, L, 256), generator=g)
+    sv = torch.randn((1, 2, L, 256), generator=g)
+    sv[:, :, 7, :8] = 3.0e5                      # one value row far beyond the float16 range
+    empty_w = torch.zeros((1, 2, 0, 64), dtype=torch.int32).view(torch.uint32).to(dev)
+    empty_s = torch.zeros((1, 2, 0, 4)).to(dev)
+    got = kquant.sdpa_fa_prefill_q8(q.to(dev), empty_w, empty_s, empty_s, empty_w, empty_s, empty_s, sk.to(dev),
+                                    sv.to(dev), 256 ** -0.5).cpu()
+    assert torch.isfinite(got).all()
+    want = qwen.causal_prefill_attention(q.numpy(), sk.numpy(), sv.clamp(-65504.0, 65504.0).numpy(), 256 ** -0.5,
+                                         past=0)
+    err = np.abs(got.numpy() - want)
+    assert err[..., 8:].max() < 2e-3 and (err[..., :8] <= 2.0 ** -10 * np.abs(want[..., :8]) + 2e-3).all()

@@ -75,6 +75,87 @@ def test_prefill_live_matches_oracle(tokens, n_comp, q_dtype):
     np.testing.assert_allclose(got.cpu().numpy(), want, rtol=2e-3, atol=2e-3)
 
 
+def _oracle_tokens(q, raw, comp, ids, sinks, tokens, *, pos0, window, ratio, raw_start=0):
+    """Oracle rows of the sampled tokens of batch entry 0 (q is BHLD): the per-token visit rules with the
+    chunk's newest ring row at pos0 + T - 1, then float64 sink attention on float16-rounded queries."""
+    T = q.shape[2]
+    out = {}
+    for t in tokens:
+        raw_rows, comp_rows = ds4.indexed_visit_rows(
+            raw_cap=raw.shape[2], n_comp=comp.shape[1], topk=ids[0, t], qpos=pos0 + t, last_pos=pos0 + T - 1,
+            window=window, ratio=ratio, raw_start=raw_start)
+        rows = np.concatenate([raw[0, 0, raw_rows].astype(np.float32).reshape(-1, 512),
+                               comp[0, comp_rows].astype(np.float32).reshape(-1, 512)], axis=0)
+        out[t] = ds4.attend_rows_f64(ds4.round_f16(q[0, :, t].astype(np.float32)), rows, sinks, 512 ** -0.5)
+    return out
+
+
+def test_prefill_live_f16_at_the_anchor_chunk():
+    """The reference's anchor chunk: 3844 tokens, 64 heads, top-512 of the pool, window 128, here from
+    position 5000 on a ring deeper than the chunk with a rotated start, and a pool that becomes visible
+    while the chunk proceeds (ids ascending; the walk stops at the first invisible one). Sampled tokens
+    against the oracle."""
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+    T, P, pos0, raw_cap, raw_start = 3844, 2300, 5000, 3900, 1234
+    rng = np.random.default_rng(2024)
+    q = rng.standard_normal((1, 64, T, 512), dtype=np.float32).astype(np.float16)
+    raw = rng.standard_normal((1, 1, raw_cap, 512), dtype=np.float32).astype(np.float16)
+    comp = rng.standard_normal((1, P, 512), dtype=np.float32).astype(np.float16)
+    ids = np.stack([np.sort(rng.choice(P, size=512, replace=False)) for _ in range(T)])[None].astype(np.int32)
+    sinks = rng.standard_normal((64,), dtype=np.float32)
+    kw = dict(pos0=pos0, window=128, ratio=4, raw_start=raw_start)
+    got = iak.indexed_mixed_attention_prefill_live_f16(_t(q), _t(raw), _t(comp), _t(ids), _t(sinks), **kw).cpu().numpy()
+    tokens = [0, 1, 63, 127, 128, 129, 1000, 1921, 2500, 3000, 3842, 3843]
+    want = _oracle_tokens(q, raw, comp, ids, sinks, tokens, **kw)
+    for t in tokens:
+        np.testing.assert_allclose(got[0, :, t], want[t], rtol=2e-3, atol=2e-3, err_msg=f"token {t}")
+    assert np.isfinite(got).all()
+
+
+def test_prefill_live_more_than_1024_keys_per_token():
+    """window + top_k beyond one workgroup's slot table: every token is split into key ranges and merged
+    with token strides."""
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+    T, P, pos0 = 300, 1500, 7000
+    rng = np.random.default_rng(7)
+    q = rng.standard_normal((1, 32, T, 512), dtype=np.float32)
+    raw = rng.standard_normal((1, 1, 900, 512), dtype=np.float32).astype(np.float16)
+    comp = rng.standard_normal((1, P, 512), dtype=np.float32).astype(np.float16)
+    ids = np.stack([np.sort(rng.choice(P, size=512, replace=False)) for _ in range(T)])[None].astype(np.int32)
+    sinks = rng.standard_normal((32,), dtype=np.float32)
+    kw = dict(pos0=pos0, window=600, ratio=4, raw_start=77)
+    got = iak.indexed_mixed_attention_prefill_live_f32(_t(q), _t(raw), _t(comp), _t(ids), _t(sinks), **kw).cpu().numpy()
+    tokens = [0, 1, 150, 298, 299]
+    want = _oracle_tokens(q, raw, comp, ids, sinks, tokens, **kw)
+    for t in tokens:
+        np.testing.assert_allclose(got[0, :, t], want[t], rtol=2e-3, atol=2e-3, err_msg=f"token {t}")
+
+
+def test_composed_reference_forms_agree_with_the_kernels():
+    """The two composed reference forms the reference module carries (:2111, :2133) against the kernels, as
+    its own tests use them (tolerance 2e-3)."""
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+    rng = np.random.default_rng(31)
+    q = rng.standard_normal((24, 16, 512), dtype=np.float32)
+    raw = rng.standard_normal((24, 512), dtype=np.float32).astype(np.float16)
+    comp = rng.standard_normal((40, 512), dtype=np.float32).astype(np.float16)
+    ids = np.stack([np.sort(rng.choice(40, size=12, replace=False)) for _ in range(24)]).astype(np.int32)
+    sinks = rng.standard_normal((16,), dtype=np.float32)
+    args = (_t(q), _t(raw), _t(comp), _t(ids), _t(sinks))
+    ref = iak.mlx_indexed_mixed_attention_prefill_reference(*args, pos0=60, window=8, ratio=4)
+    got = iak.indexed_mixed_attention_prefill(*args, pos0=60, window=8, ratio=4)
+    np.testing.assert_allclose(got.cpu().numpy(), ref.cpu().numpy(), rtol=2e-3, atol=2e-3)
+    np.testing.assert_allclose(ref.cpu().numpy(), ds4.indexed_mixed_attention_prefill_reference(
+        q, raw, comp, ids, sinks, pos0=60, window=8, ratio=4), rtol=1e-4, atol=1e-5)
+    one = iak.mlx_selected_rows_attention_reference(_t(q[0]), _t(raw), _t(comp), _t(ids[0]), _t(sinks))
+    dec = iak.indexed_mixed_attention_decode(_t(q[0]), _t(raw), _t(comp), _t(ids[0]), _t(sinks), pos0=40 * 4 + 23,
+                                             window=128)
+    np.testing.assert_allclose(dec.cpu().numpy(), one.cpu().numpy(), rtol=2e-3, atol=2e-3)
+
+
 def test_prefill_live_negative_and_stop_ids_offset_chunk_and_ring():
     """Negative ids are skipped, the first invisible id ends the walk, the chunk starts at pos0 > 0 and the
     ring is deeper than the chunk with a rotated start (reference :423-505)."""
@@ -157,6 +238,27 @@ def test_indexer_scores_tiled_live(dtype):
         iak.indexer_scores_tiled_live(_t(q, torch.float16), _t(w), _t(comp), pos0=0)
     with pytest.raises(ValueError, match="weights must be float32"):
         iak.indexer_scores_tiled_live(_t(q), _t(w, torch.float16), _t(comp), pos0=0)
+
+
+def test_indexer_scores_tiled_live_at_the_anchor_chunk():
+    """3844 tokens x 961 pool rows x 64 heads, float16 operands (the served form); sampled tokens against the
+    oracle, each as a one-token chunk at its own position."""
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+    T, P, H, pos0 = 3844, 961, 64, 0
+    rng = np.random.default_rng(11)
+    q = rng.standard_normal((1, H, T, 128), dtype=np.float32).astype(np.float16)
+    comp = rng.standard_normal((1, P, 128), dtype=np.float32).astype(np.float16)
+    w = (rng.standard_normal((1, T, H), dtype=np.float32) * (H ** -0.5) * (128 ** -0.5)).astype(np.float32)
+    got = iak.indexer_scores_tiled_live(_t(q), _t(w), _t(comp), pos0=pos0, ratio=4).cpu().numpy()
+    assert got.shape == (1, T, P)
+    for t in (0, 2, 3, 4, 500, 1921, 3000, 3843):
+        want = ds4.indexer_scores_tiled_live(q[:, :, t:t + 1].astype(np.float32), w[:, t:t + 1],
+                                             comp.astype(np.float32), pos0=pos0 + t, ratio=4)[0, 0]
+        inf = np.isinf(want)
+        assert inf.sum() == P - min((pos0 + t + 1) // 4, P)
+        assert (np.isinf(got[0, t]) == inf).all()
+        np.testing.assert_allclose(got[0, t][~inf], want[~inf], rtol=1e-4, atol=1e-4, err_msg=f"token {t}")
 
 
 def test_indexer_scores_tiled_live_f16_operands_bit_identical():

@@ -43,6 +43,8 @@ def _affine_cache(rng, B, Hkv, N, sb_dtype):
     (1, 16, 2, 257, torch.bfloat16),
     (2, 8, 4, 1000, torch.float16),
     (1, 16, 2, 4099, torch.bfloat16),
+    (1, 16, 2, 8192, torch.bfloat16),      # the depth from which the reference engages this operator
+    (1, 16, 2, 37000, torch.bfloat16),     # BASELINE config 3 depth, scales as served (bfloat16)
     (1, 4, 4, 300, torch.float32),
     (1, 32, 2, 129, torch.float32),
 ])

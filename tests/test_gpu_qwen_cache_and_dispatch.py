@@ -61,6 +61,43 @@ def test_quantized_cache_appends_and_grows():
     assert torch.equal(sk[0].view(torch.int32), k[0].view(torch.int32)) and int(sv[2].shape[2]) == total
 
 
+def test_cache_views_reach_the_kernels_without_a_copy():
+    """The cache grows in 256-row blocks and hands out its first `offset` rows of every head: views that are
+    not contiguous with two KV heads. The operators must read them where they lie (row capacity as an
+    argument), not copy the whole cache per token, and give the bits of the contiguous form."""
+    from moespresso_amd.runtime.qwen import kquant
+
+    g = torch.Generator().manual_seed(5)
+    cache = kquant.QuantizedKVCache()
+    k, v = cache.update_and_fetch(torch.randn((1, 2, 300, 256), generator=g).to(_dev()),
+                                  torch.randn((1, 2, 300, 256), generator=g).to(_dev()))
+    assert not k[0].is_contiguous() and int(cache.keys[0].shape[2]) == 512
+    handed, rows = kquant._cache_operands(k + v, 300)
+    assert rows == 512
+    for given, view, buf in zip(handed, k + v, cache.keys + cache.values):
+        assert given is view and given.data_ptr() == buf.data_ptr()
+    # a layout that is no leading-row view falls back to one dense copy
+    odd, rows = kquant._cache_operands(tuple(t.flip(2) for t in k + v), 300)
+    assert rows == 300 and all(t.is_contiguous() for t in odd)
+
+    q = torch.randn((1, 16, 1, 256), generator=g).to(_dev())
+    dense = tuple(t.contiguous() for t in k + v)
+    got = kquant.sdpa_decode_q8(q, *k, *v, 256 ** -0.5)
+    assert torch.equal(got, kquant.sdpa_decode_q8(q, *dense, 256 ** -0.5))
+    qs = torch.randn((1, 16, 40, 256), generator=g).to(_dev())
+    sk = torch.randn((1, 2, 40, 256), generator=g).to(_dev())
+    got = kquant.sdpa_fa_prefill_q8(qs, *k, *v, sk, 2 * sk, 256 ** -0.5)
+    assert torch.equal(got, kquant.sdpa_fa_prefill_q8(qs, *dense, sk, 2 * sk, 256 ** -0.5))
+    # Q8_0 form: leading rows of a larger buffer
+    kc = torch.randint(-127, 128, (2, 2, 512, 256), generator=g, dtype=torch.int8).to(_dev())
+    ks = (torch.rand((2, 2, 512, 8), generator=g) * 0.03).half().to(_dev())
+    q0 = torch.randn((2, 16, 256), generator=g).to(_dev())
+    got = kquant.sdpa_decode_q8_0(q0, kc[:, :, :301], ks[:, :, :301], kc[:, :, :301], ks[:, :, :301], 256 ** -0.5)
+    want = kquant.sdpa_decode_q8_0(q0, kc[:, :, :301].contiguous(), ks[:, :, :301].contiguous(),
+                                   kc[:, :, :301].contiguous(), ks[:, :, :301].contiguous(), 256 ** -0.5)
+    assert torch.equal(got, want)
+
+
 class _Block(torch.nn.Module):
     """A small gated attention block with the attribute names the wrapper uses (random weights)."""
 

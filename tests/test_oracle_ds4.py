@@ -505,3 +505,121 @@ def test_tiled_live_scores_closed_form_and_visibility():
                     assert abs(got[b, t, c] - want) < 1e-9
                 else:
                     assert got[b, t, c] == -np.inf
+
+
+def test_round_bf16_and_f16_match_torch_casts():
+    # a truncating or round-half-up restatement would pass idempotence; the library cast pins the rule
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, 20000).astype(np.float32)
+    ties = (np.arange(1, 4097, dtype=np.uint32) << 16 | 0x8000).view(np.float32)          # exact bf16 midpoints
+    special = np.array([0.0, -0.0, np.inf, -np.inf, 1e-45, -1e-40, 3.3895314e38, 65504.0, 65520.0, 65519.99],
+                       dtype=np.float32)
+    for a in (x, ties, -ties, special):
+        want = torch.from_numpy(a).to(torch.bfloat16).to(torch.float32).numpy()
+        np.testing.assert_array_equal(ds4.round_bf16(a).view(np.uint32), want.view(np.uint32))
+        want16 = torch.from_numpy(a).to(torch.float16).to(torch.float32).numpy()
+        np.testing.assert_array_equal(ds4.round_f16(a).view(np.uint32), want16.view(np.uint32))
+    assert np.isnan(ds4.round_bf16(np.array([np.nan], np.float32))).all()
+
+
+def _walk_token(raw, comp, ids, qpos, newest_pos, window, ratio, raw_start):
+    """Rows one query visits, by absolute position (independent of ds4.indexed_visit_rows): the ring holds
+    the raw_cap newest positions ending at newest_pos, position p at row (raw_start + p - oldest) % raw_cap."""
+    raw_cap = raw.shape[0]
+    oldest = newest_pos - raw_cap + 1
+    rows = []
+    for p in range(max(0, oldest), newest_pos + 1):
+        if p > qpos or (window and p <= qpos - window):
+            continue
+        rows.append(raw[(raw_start + p - oldest) % raw_cap])
+    visible = comp.shape[0] if ratio == 0 else min((qpos + 1) // ratio, comp.shape[0])
+    for i in ids:
+        if i < 0:
+            continue
+        if i >= visible:
+            break
+        rows.append(comp[i])
+    return np.stack(rows) if rows else np.zeros((0, raw.shape[1]), np.float32)
+
+
+def test_indexed_prefill_against_an_independent_walk_and_the_composed_reference_form():
+    rng = np.random.default_rng(77)
+    T, H, P = 37, 4, 30
+    q = (rng.standard_normal((T, H, 512)) * 0.4).astype(np.float32)
+    comp = (rng.standard_normal((P, 512)) * 0.5).astype(np.float16)
+    sinks = rng.standard_normal(H).astype(np.float32)
+    for pos0, raw_cap, window, raw_start, ratio in ((0, 37, 16, 0, 4), (50, 37, 128, 11, 4), (3, 64, 8, 63, 4),
+                                                    (90, 20, 0, 5, 0)):
+        raw = (rng.standard_normal((raw_cap, 512)) * 0.5).astype(np.float16)
+        ids = np.stack([np.sort(rng.choice(P, 9, replace=False)) for _ in range(T)]).astype(np.int32)
+        ids[3, 2] = -1
+        got = ds4.indexed_mixed_attention_prefill(q, raw, comp, ids, sinks, pos0=pos0, window=window, ratio=ratio,
+                                                  raw_start=raw_start)
+        newest = pos0 + T - 1
+        for t in range(T):
+            rows = _walk_token(raw.astype(np.float32), comp.astype(np.float32), ids[t].tolist(), pos0 + t, newest,
+                               window, ratio, raw_start).astype(np.float64)
+            qh = torch.from_numpy(q[t]).to(torch.float16).to(torch.float64)
+            logits = torch.cat([qh @ torch.from_numpy(rows).T * 512 ** -0.5,
+                                torch.from_numpy(sinks.astype(np.float64))[:, None]], dim=1)
+            prob = torch.softmax(logits, dim=1)[:, :-1]
+            want = (prob @ torch.from_numpy(rows)).numpy() if rows.shape[0] else np.zeros((H, 512))
+            np.testing.assert_allclose(got[t], want, rtol=1e-12, atol=1e-12, err_msg=f"{pos0} {t}")
+        if raw_start == 0 and ratio != 0:
+            # ascending ids: the composed form's filter selects the rows the kernel's stop rule does; its
+            # float16 sinks move the result by at most the rounding of the sink logit
+            ref = ds4.indexed_mixed_attention_prefill_reference(q, raw, comp, ids, sinks, pos0=pos0, window=window,
+                                                                ratio=ratio)
+            np.testing.assert_allclose(ref, got, rtol=0, atol=2e-3)
+    # unsorted ids: the kernel stops at the first invisible id, the composed form only drops it
+    raw = (rng.standard_normal((8, 512)) * 0.5).astype(np.float16)
+    ids = np.tile(np.array([[1, 29, 0]], np.int32), (8, 1))          # visible = (qpos+1)//4 <= 4 < 29
+    stop = ds4.indexed_mixed_attention_prefill(q[:8], raw, comp, ids, sinks, pos0=8, window=128, ratio=4)
+    filt = ds4.indexed_mixed_attention_prefill_reference(q[:8], raw, comp, ids, sinks, pos0=8, window=128, ratio=4)
+    only_first = ds4.indexed_mixed_attention_prefill(q[:8], raw, comp, ids[:, :1], sinks, pos0=8, window=128, ratio=4)
+    both = ds4.indexed_mixed_attention_prefill(q[:8], raw, comp, ids[:, [0, 2]], sinks, pos0=8, window=128, ratio=4)
+    np.testing.assert_array_equal(stop, only_first)
+    np.testing.assert_allclose(filt, both, rtol=0, atol=2e-3)
+    assert np.abs(filt - stop).max() > 1e-2
+
+
+def test_fused_decode_prep_all_tie_integer_and_row_parts():
+    # reference tests/test_deepseek_v4_decode_attention_kernel.py:215-243: equal scores select arange(topk)
+    inv = ds4.rope_inverse_frequencies(64, ds4.DS4_COMPRESS_ROPE_BASE, ds4.DS4_YARN).astype(np.float32)
+    H, N, K = 8, 50, 7
+    q = np.zeros((H, 128), np.float32)
+    pooled = np.ones((N, 128), np.float32)
+    w = np.ones(H, np.float32)
+    kv = np.zeros(512, np.float16)
+    params = np.array([100, 0], np.int32)
+    sel, row, scores = ds4.fused_decode_prep(q, pooled, w, kv, inv, params, scale=128 ** -0.5, topk=K)
+    np.testing.assert_array_equal(sel, np.arange(K))
+    assert np.all(scores == 0) and np.all(row == 0)
+    # q = ones: the QAT row is [12, 0, ...] exactly (Hadamard of ones), so score(r) = sum_h w_h relu(12 p_r0) scale
+    # computable by hand; distinct integers in column 0 give a known order, equal ones tie to the lower row
+    q = np.ones((H, 128), np.float32)
+    rng = np.random.default_rng(3)
+    col0 = rng.integers(-3, 6, N).astype(np.float32)
+    pooled = np.zeros((N, 128), np.float32)
+    pooled[:, 0] = col0
+    pooled[:, 1:] = rng.integers(-2, 3, (N, 127))                 # multiplied by exact zeros of the QAT row
+    w = (rng.integers(1, 5, H) * 0.25).astype(np.float32)
+    sel, _, scores = ds4.fused_decode_prep(q, pooled, w, kv, inv, params, scale=0.5, topk=K)
+    by_hand = np.maximum(12.0 * col0.astype(np.float64), 0.0) * 0.5 * w.astype(np.float64).sum()
+    np.testing.assert_allclose(scores, by_hand, rtol=0, atol=1e-9)
+    order = np.lexsort((np.arange(N), -by_hand))[:K]
+    thr = by_hand[order[-1]]
+    above = np.nonzero(by_hand > thr)[0]
+    ties = np.nonzero(by_hand == thr)[0][:K - above.size]
+    np.testing.assert_array_equal(sel, np.concatenate([above, ties]))   # emission: above ascending, then ties
+    # prepared row = FP8 round trip of the first 448 columns + rope of the last 64 at float16 rounding
+    kv = (rng.standard_normal(512) * 0.3).astype(np.float16)
+    _, row, _ = ds4.fused_decode_prep(q, pooled, w, kv, inv, np.array([3844, 0], np.int32), scale=0.5, topk=K)
+    head = ds4.fp8_kv_roundtrip(kv.astype(np.float32))[:448].astype(np.float16)
+    np.testing.assert_array_equal(row[:448].view(np.uint16), head.view(np.uint16))
+    # (float16 rounding of cos/sin, of the four products and of the two sums: within 2e-3 of the float64 rotation)
+    x = kv[448:].astype(np.float64).reshape(32, 2)
+    ang = 3844.0 * inv.astype(np.float64)
+    want = np.stack([x[:, 0] * np.cos(ang) - x[:, 1] * np.sin(ang), x[:, 0] * np.sin(ang) + x[:, 1] * np.cos(ang)], 1)
+    np.testing.assert_allclose(row[448:].astype(np.float64), want.reshape(-1), rtol=0, atol=2e-3)
+    assert np.abs(row[448:].astype(np.float64) - kv[448:].astype(np.float64)).max() > 0.05    # it did rotate

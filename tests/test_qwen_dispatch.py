@@ -111,5 +111,30 @@ def test_fixed_decode_state_helpers_match_oracle():
     scores = rng.standard_normal((1, 3, 9)).astype(np.float32)
     got = fds.pad_scores_to_capacity(torch.from_numpy(scores), params).numpy()
     np.testing.assert_array_equal(got, ds4.pad_scores_to_capacity(scores, 5))
+    # the reference's call sites pass their array module first (fixed_decode_state.py:186,198 called as
+    # decode_step_params(mx, offset=…, pool_rows=…) and pad_scores_to_capacity(mx, scores, params))
+    np.testing.assert_array_equal(fds.decode_step_params(torch, offset=41, pool_rows=5).numpy(), params.numpy())
+    np.testing.assert_array_equal(fds.pad_scores_to_capacity(torch, torch.from_numpy(scores), params).numpy(), got)
+    with pytest.raises(TypeError):
+        fds.pad_scores_to_capacity(torch.from_numpy(scores))
     with pytest.raises(ValueError, match="int32"):
         fds.pad_scores_to_capacity(torch.from_numpy(scores), params.float())
+
+
+def test_row_capacity_of_cache_views():
+    from moespresso_amd.runtime.qwen.kquant import _cache_operands, _row_capacity
+
+    buf = torch.zeros((2, 2, 512, 64))
+    assert _row_capacity(buf[:, :, :300], 300) == 512          # leading rows of every head
+    assert _row_capacity(buf, 512) == 512
+    assert _row_capacity(buf[:, :, :300].contiguous(), 300) == 300
+    assert _row_capacity(buf[:, :, 5:305], 300) == 512         # same strides from another first row
+    assert _row_capacity(buf[:, :1, :300], 300) == 1024        # one head of two: the batch stride is the capacity
+    assert _row_capacity(buf[:1, :1, :300], 300) == 300
+    assert _row_capacity(buf.transpose(1, 2)[:, :300], 300) is None
+    assert _row_capacity(buf[:, :, :300, ::2], 300) is None
+    a, b = buf[:, :, :300], torch.zeros((2, 2, 768, 4))[:, :, :300]
+    same, rows = _cache_operands((a, a), 300)
+    assert rows == 512 and same[0] is a
+    mixed, rows = _cache_operands((a, b), 300)                 # capacities differ: dense copies
+    assert rows == 300 and all(t.is_contiguous() for t in mixed)
