@@ -34,9 +34,24 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the dominant kernel at batch 16 (FETCH_SIZE + WRITE_SIZE of rocprofv3 --pmc, scaled by
-# the same counters' reading for a 1 GiB elementwise kernel; profiles/bench_sparse_decode_layer_hbm_counters.txt)
-SPLIT_TRAFFIC_BYTES_B16 = 58_490_000
+COUNTERS_FILE = os.path.join(ROOT, "profiles", "bench_sparse_decode_layer_hbm_counters.txt")
+
+
+def measured_traffic_bytes(kernel_prefix: str, workgroups: int):
+    """HBM bytes per launch of one kernel as the committed rocprofv3 counter summary reports them (FETCH_SIZE +
+    WRITE_SIZE, each scaled by the same counter's reading for a copy kernel of known size); None when the
+    summary does not hold that launch shape."""
+    try:
+        with open(COUNTERS_FILE) as f:
+            for line in f:
+                if not line.startswith(kernel_prefix):
+                    continue
+                cols = line[44:].split()
+                if len(cols) >= 7 and int(cols[0]) == workgroups:
+                    return int(round(float(cols[6]) * 1e6))
+    except (OSError, ValueError):
+        pass
+    return None
 
 # workload constants (BASELINE configs 4 and 5)
 N_IDX_HEADS, IDX_DIM, N_KEYS, TOPK = 64, 128, 32768, 2048
@@ -60,7 +75,7 @@ def make_set(batch: int, dev, gen):
     return dict(qi=qi, keys=keys, kscale=kscale, w=w, q=q, kv=kv)
 
 
-def cpu_baseline(seconds_budget: float = 15.0):
+def cpu_baseline(seconds_budget: float = 10.0, threads: int | None = None):
     """The NumPy oracle on one sequence of the same step; scaled to the 16-sequence layer."""
     from oracle import ds4
 
@@ -68,7 +83,7 @@ def cpu_baseline(seconds_budget: float = 15.0):
         from threadpoolctl import threadpool_limits
     except Exception:  # pragma: no cover
         threadpool_limits = None
-    cores = min(16, os.cpu_count() or 1)
+    cores = min(16, os.cpu_count() or 1) if threads is None else threads
     rng = np.random.default_rng(0)
     qi = ds4.round_bf16(rng.standard_normal((1, N_IDX_HEADS, IDX_DIM), dtype=np.float32))
     k32 = rng.standard_normal((1, N_KEYS, IDX_DIM), dtype=np.float32)
@@ -105,6 +120,59 @@ def cpu_baseline(seconds_budget: float = 15.0):
         "sample": f"{reps} repeats of one sequence (1/16 of the layer: 32768-key indexer + top-2048 + 2176-row "
                   f"MLA decode), NumPy oracle with {cores} BLAS threads, scaled x16",
     }
+
+
+def cpu_other_configs():
+    """BASELINE configs 2 and 3 on the host through the NumPy oracle, on bounded samples (a reported baseline):
+    config 3 whole at batch 1; config 2 on 128 of the 4096 query rows (the last ones: the deepest causal rows),
+    scaled by the ratio of causal FLOPs."""
+    from oracle import qwen
+
+    try:
+        from threadpoolctl import threadpool_limits
+    except Exception:  # pragma: no cover
+        threadpool_limits = None
+    cores = min(16, os.cpu_count() or 1)
+    rng = np.random.default_rng(0)
+    out = {}
+    ctx = threadpool_limits(limits=cores) if threadpool_limits else None
+    try:
+        N = 37000
+        kc, ks = qwen.q8_0_quantize(rng.standard_normal((1, 2, N, 256), dtype=np.float32))
+        vc, vs = qwen.q8_0_quantize(rng.standard_normal((1, 2, N, 256), dtype=np.float32))
+        q = rng.standard_normal((1, 16, 1, 256), dtype=np.float32)
+
+        def decode():
+            return qwen.gqa_decode_attention(q, qwen.q8_0_dequantize(kc, ks), qwen.q8_0_dequantize(vc, vs), 256 ** -0.5)
+
+        t0 = time.perf_counter()
+        decode()
+        reps = 1
+        if time.perf_counter() - t0 < 1.0:  # fast host: the first call was the warm-up
+            t0 = time.perf_counter()
+            reps = 0
+            while reps < 20 and time.perf_counter() - t0 < 3.0:
+                decode()
+                reps += 1
+        out["config3_B1_us"] = round((time.perf_counter() - t0) / max(reps, 1) * 1e6, 1)
+        out["config3_sample"] = f"{reps} repeats, dequantise + float64 attention over 37000 keys, batch 1"
+        L, past, rows = 4096, 32768, 128
+        k = (0.5 * rng.standard_normal((1, 2, past + L, 256), dtype=np.float32))
+        v = (0.5 * rng.standard_normal((1, 2, past + L, 256), dtype=np.float32))
+        qs = (0.5 * rng.standard_normal((1, 16, rows, 256), dtype=np.float32))
+        t0 = time.perf_counter()
+        qwen.causal_prefill_attention(qs, k, v, 256 ** -0.5, past=past + L - rows)
+        dt = time.perf_counter() - t0
+        sample_flops = 4.0 * 256 * 16 * sum(past + L - rows + i + 1 for i in range(rows))
+        full_flops = 4.0 * 256 * 16 * (L * past + L * (L + 1) / 2)
+        out["config2_ms"] = round(dt * full_flops / sample_flops * 1e3, 1)
+        out["config2_sample"] = f"the last {rows} of {L} query rows once ({dt:.2f} s), scaled by causal FLOPs x{full_flops / sample_flops:.1f}"
+    finally:
+        if ctx is not None:
+            ctx.__exit__(None, None, None)
+    out["cores"] = cores
+    out["kind"] = "port"
+    return out
 
 
 def cpu_config1():
@@ -151,6 +219,36 @@ def bench_prefill(dev, gen, reps=10, warmup=20):
     return {"ms": round(ms, 4), "TFLOPs": round(tf, 1), "peak_TFLOPs": 2500.0, "frac": round(tf / 2500.0, 4),
             "tokens_per_s": round(L / (ms * 1e-3), 1), "bound": "mfma",
             "workload": "causal prefill, 4096 new x 32768 prefix, 16q/2kv heads, D=256, bf16 (BASELINE config 2)"}
+
+
+def bench_prefill_q8(dev, gen, reps=6, warmup=10):
+    """The reference's own prefill callable at the same depth: 4096 float32 queries over a 32768-token affine
+    8-bit prefix plus the dense chunk (full_attention.py:372 call site)."""
+    from moespresso_amd import _lib
+    from moespresso_amd.runtime.qwen import kquant
+
+    L, past = 4096, 32768
+    q = 0.5 * torch.randn((1, 16, L, 256), device=dev, generator=gen)
+    pk = kquant.quantize(0.5 * torch.randn((1, 2, past, 256), device=dev, generator=gen))
+    pv = kquant.quantize(0.5 * torch.randn((1, 2, past, 256), device=dev, generator=gen))
+    sk = 0.5 * torch.randn((1, 2, L, 256), device=dev, generator=gen)
+    sv = 0.5 * torch.randn((1, 2, L, 256), device=dev, generator=gen)
+    nbytes = int(_lib.lib().mspr_sdpa_fa_prefill_q8_workspace_bytes(1, 16, 2, L, past))
+    ws = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=dev)
+    run = lambda: kquant.sdpa_fa_prefill_q8(q, *pk, *pv, sk, sv, 256 ** -0.5, workspace=ws)
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    _lib.profile_enable("flash_prefill")
+    for _ in range(reps):
+        run()
+    torch.cuda.synchronize()
+    ms = float(np.mean(_lib.profile_collect("flash_prefill")))
+    _lib.profile_enable()
+    flops = 4.0 * 256 * 16 * (L * past + L * (L + 1) / 2)
+    tf = flops / (ms * 1e-3) / 1e12
+    return {"ms": round(ms, 4), "TFLOPs": round(tf, 1), "frac": round(tf / 2500.0, 4),
+            "workload": "sdpa_fa_prefill_q8: 4096 new x 32768-token affine 8-bit prefix, float32 queries, float16 MFMA"}
 
 
 def bench_q8_decode(dev, gen, reps=40):
@@ -238,6 +336,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--sets", type=int, default=8, help="distinct buffer sets rotated through (cold caches)")
+    ap.add_argument("--regions", type=int, default=9, help="timed regions of --steps steps each; the median is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one elementwise kernel that reads 1 GiB and writes 1 GiB (scale for HBM counters)")
@@ -305,10 +404,16 @@ def main() -> int:
 
     replay_steps(W)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    replay_steps(K)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    # a timed region is exactly K steps between two synchronisations; short regions (the driver's K = 20 is about
+    # a millisecond) are repeated and the median region is reported
+    regions = []
+    for _ in range(args.regions):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        replay_steps(K)
+        torch.cuda.synchronize()
+        regions.append(time.perf_counter() - t0)
+    elapsed = float(np.median(regions))
     ms_per_step = elapsed / K * 1e3
 
     # per-kernel GPU durations: same steps, eager, HIP events around each kernel on its launch stream
@@ -322,6 +427,7 @@ def main() -> int:
 
     split_us = kernel_us["sparse_split"]
     achieved = MLA_BYTES_PER_SEQ * B / (split_us * 1e-6) / 1e9
+    operator_us = split_us + kernel_us["sparse_merge"]
     roofline = {
         "kernel": "sparse_attn_split_kernel<bf16,576>",
         "bound": "hbm",
@@ -329,9 +435,12 @@ def main() -> int:
         "peak": HBM_PEAK_GBS,
         "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4),
-        "traffic": SPLIT_TRAFFIC_BYTES_B16 if B == 16 else None,
+        "traffic": measured_traffic_bytes("sparse_attn_split_kernel<2, 576", B * 16) if B == 16 else None,
         "algorithmic_bytes_per_launch": MLA_BYTES_PER_SEQ * B,
         "kernel_us": round(split_us, 2),
+        # the whole operator (split + merge launches) against the same algorithmic bytes
+        "operator_us": round(operator_us, 2),
+        "operator_frac": round(MLA_BYTES_PER_SEQ * B / (operator_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
     }
     # the same kernels at the smaller batches of the configuration (first sequences of the same buffers)
     by_batch = {}
@@ -364,9 +473,12 @@ def main() -> int:
         "kernel_us": {k: round(v, 2) for k, v in kernel_us.items()},
         "kernel_us_by_batch": by_batch,
         "prefill": None if args.headline_only else bench_prefill(dev, gen),
+        "prefill_q8": None if args.headline_only else bench_prefill_q8(dev, gen),
         "q8_decode": None if args.headline_only else bench_q8_decode(dev, gen),
         "ds4_prefill": None if args.headline_only else bench_ds4_prefill(dev, gen),
         "cpu_config1": None if args.no_cpu_baseline else cpu_config1(),
+        "cpu_configs_2_3": None if args.no_cpu_baseline else cpu_other_configs(),
+        "cpu_baseline_1thread": None if args.no_cpu_baseline else cpu_baseline(seconds_budget=6.0, threads=1),
         "indexer_fp8_GBps": round(IDX_BYTES_PER_SEQ * B / (kernel_us["indexer_fp8"] * 1e-6) / 1e9, 1),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
         "buffer_sets": R,
@@ -386,6 +498,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": K,
         "warmup": W,
+        "timed_regions": args.regions,
         "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": False,
         "scaling": "weak",
