@@ -91,6 +91,20 @@ int mspr_fused_decode_prep(const void* q_idx, int q_dtype, int n_heads, const fl
                            const float* inv_freq, const int32_t* params, float scale, int topk,
                            int32_t* sel, void* row_out, float* scores, void* stream);
 
+/* fused_decode_prep over a fixed-capacity pool: pooled_qat holds `capacity` rows of which the first
+ * params[2] are in use; params: int32 [position, ring write index, pool rows in use] ON THE DEVICE, so a
+ * launch recorded into a HIP graph follows the pool as it grows (the caller appends rows to the buffer
+ * and rewrites params between replays). Rows not in use score -inf; with topk <= rows in use the
+ * selection and its order equal mspr_fused_decode_prep on the first params[2] rows bit for bit, with
+ * fewer rows in use the surplus ids name unused rows, which mspr_fused_decode_sdpa_fixed skips.
+ * The counterpart of the fixed-capacity decode state, runtime/deepseek_v4/fixed_decode_state.py:186-206
+ * (decode_step_params, pad_scores_to_capacity) and :215-288 (capacity buffers of the derived caches).
+ * scores: f32 [capacity]; 0 < topk < capacity. */
+int mspr_fused_decode_prep_fixed(const void* q_idx, int q_dtype, int n_heads, const float* pooled_qat,
+                                 int64_t capacity, const float* weights, const void* kv_row,
+                                 const float* inv_freq, const int32_t* params, float scale, int topk,
+                                 int32_t* sel, void* row_out, float* scores, void* stream);
+
 /* Extension (BASELINE config 4): batched lightning-indexer scores with FP8 keys.
  *   scores[b,r] = sum_h w[b,h] * relu(q[b,h] . e4m3(keys[b,r])) * key_scales[b,r]
  * q: bf16 [batch,n_heads,128] (n_heads <= 64); keys: E4M3FN bytes [batch,n_rows,128];
@@ -163,6 +177,16 @@ int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* window, int w
                            int n_sel, const void* sinks, const float* inv_freq, const int32_t* params,
                            float scale, void* out, void* workspace, size_t workspace_bytes,
                            void* stream);
+
+/* fused_decode_sdpa over a fixed-capacity pool: pooled holds `capacity` rows, params is int32
+ * [position, ring write index, pool rows in use] on the device; ids in sel that are negative or name a
+ * row not in use are skipped. Same arithmetic as mspr_fused_decode_sdpa otherwise (fixed-capacity decode
+ * state, fixed_decode_state.py:186-206). */
+int mspr_fused_decode_sdpa_fixed(const void* q, int n_heads, const void* window, int window_rows,
+                                 const void* row, const void* pooled, int64_t capacity, const int32_t* sel,
+                                 int n_sel, const void* sinks, const float* inv_freq, const int32_t* params,
+                                 float scale, void* out, void* workspace, size_t workspace_bytes,
+                                 void* stream);
 
 /* Extension (BASELINE config 5): batched sparse multi-head latent decode attention.
  * Every head of batch b attends rows kv[b, rows[b, :]] of a shared latent cache; K is the whole

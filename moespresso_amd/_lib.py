@@ -34,6 +34,12 @@ SIGNATURES = {
     "mspr_fused_decode_prep": (
         c_int, [c_void_p, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
                 c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "mspr_fused_decode_prep_fixed": (
+        c_int, [c_void_p, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
+                c_float, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "mspr_fused_decode_sdpa_fixed": (
+        c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_void_p,
+                c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_indexer_scores_fp8": (
         c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_void_p, c_void_p]),
     "mspr_indexer_q_qat_live": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),

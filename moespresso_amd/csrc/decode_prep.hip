@@ -6,14 +6,14 @@
 
 int mspr_launch_scores_f32(const void* q, int q_dtype, int n_heads, const float* pooled, int64_t n_rows,
                            const float* weights, float scale, float* scores, bool stage_half, const void* kv_row,
-                           const float* inv_freq, const int32_t* params, void* row_out, hipStream_t st);
+                           const float* inv_freq, const int32_t* params, void* row_out, const int32_t* valid_rows,
+                           hipStream_t st);
 int mspr_launch_topk(const float* scores, int64_t score_stride, int batch, int64_t n_rows, int topk, int32_t* sel,
                      hipStream_t st);
 
-extern "C" int mspr_fused_decode_prep(const void* q_idx, int q_dtype, int n_heads, const float* pooled_qat,
-                                      int64_t n_rows, const float* weights, const void* kv_row,
-                                      const float* inv_freq, const int32_t* params, float scale, int topk,
-                                      int32_t* sel, void* row_out, float* scores, void* stream) {
+static int decode_prep(const void* q_idx, int q_dtype, int n_heads, const float* pooled_qat, int64_t n_rows,
+                       const float* weights, const void* kv_row, const float* inv_freq, const int32_t* params,
+                       float scale, int topk, int32_t* sel, void* row_out, float* scores, bool fixed, void* stream) {
   MSPR_REQUIRE(q_idx && pooled_qat && weights && kv_row && inv_freq && params && sel && row_out && scores,
                "fused_decode_prep: null pointer");
   MSPR_REQUIRE(n_heads >= 1 && n_heads <= 64, "fused_decode_prep: q_idx must carry between 1 and 64 heads");
@@ -25,7 +25,23 @@ extern "C" int mspr_fused_decode_prep(const void* q_idx, int q_dtype, int n_head
                "fused_decode_prep: q_idx, pooled_qat, kv_row and row_out must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   int rc = mspr_launch_scores_f32(q_idx, q_dtype, n_heads, pooled_qat, n_rows, weights, scale, scores, true, kv_row,
-                                  inv_freq, params, row_out, st);
+                                  inv_freq, params, row_out, fixed ? params + 2 : nullptr, st);
   if (rc != MSPR_OK) return rc;
   return mspr_launch_topk(scores, n_rows, 1, n_rows, topk, sel, st);
+}
+
+extern "C" int mspr_fused_decode_prep(const void* q_idx, int q_dtype, int n_heads, const float* pooled_qat,
+                                      int64_t n_rows, const float* weights, const void* kv_row,
+                                      const float* inv_freq, const int32_t* params, float scale, int topk,
+                                      int32_t* sel, void* row_out, float* scores, void* stream) {
+  return decode_prep(q_idx, q_dtype, n_heads, pooled_qat, n_rows, weights, kv_row, inv_freq, params, scale, topk, sel,
+                     row_out, scores, false, stream);
+}
+
+extern "C" int mspr_fused_decode_prep_fixed(const void* q_idx, int q_dtype, int n_heads, const float* pooled_qat,
+                                            int64_t capacity, const float* weights, const void* kv_row,
+                                            const float* inv_freq, const int32_t* params, float scale, int topk,
+                                            int32_t* sel, void* row_out, float* scores, void* stream) {
+  return decode_prep(q_idx, q_dtype, n_heads, pooled_qat, capacity, weights, kv_row, inv_freq, params, scale, topk,
+                     sel, row_out, scores, true, stream);
 }

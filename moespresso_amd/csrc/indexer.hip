@@ -341,7 +341,8 @@ __global__ __launch_bounds__(kScoreThreads) void scores_f32_kernel(const void* _
                                                                    const uint16_t* __restrict__ kv_row,
                                                                    const float* __restrict__ inv_freq,
                                                                    const int32_t* __restrict__ params,
-                                                                   uint16_t* __restrict__ row_out) {
+                                                                   uint16_t* __restrict__ row_out,
+                                                                   const int32_t* __restrict__ valid_rows) {
   __shared__ float qbuf[64 * kQPitch];
   __shared__ float wbuf[64];
   __shared__ float ptab[kPow2TabLen];
@@ -499,7 +500,9 @@ __global__ __launch_bounds__(kScoreThreads) void scores_f32_kernel(const void* _
       sum += mul_rn(mul_rn(fmaxf(acc1[i], 0.0f), scale), wl[1][i]);
     }
     sum += __shfl_xor(sum, 32, MSPR_WAVE);
-    if (g == 0 && row < n_rows) scores[row] = sum;
+    // fixed-capacity form: the pool buffer holds n_rows rows of which the first *valid_rows are in use (a
+    // count that lives on the device, so that a captured launch follows a growing pool); the rest score -inf
+    if (g == 0 && row < n_rows) scores[row] = (valid_rows && row >= (int64_t)valid_rows[0]) ? -__builtin_inff() : sum;
   }
 }
 
@@ -534,7 +537,8 @@ extern "C" int mspr_indexer_q_qat_live(const float* q, int64_t n_rows, float* ou
 // kv_row (with inv_freq, params, row_out) may be null: no prepared KV row in this launch
 int mspr_launch_scores_f32(const void* q, int q_dtype, int n_heads, const float* pooled, int64_t n_rows,
                            const float* weights, float scale, float* scores, bool stage_half, const void* kv_row,
-                           const float* inv_freq, const int32_t* params, void* row_out, hipStream_t st) {
+                           const float* inv_freq, const int32_t* params, void* row_out, const int32_t* valid_rows,
+                           hipStream_t st) {
   int64_t n_tiles = (n_rows + 31) / 32;
   int64_t blocks = (n_tiles + kScoreWaves - 1) / kScoreWaves;
   if (blocks > 2048) blocks = 2048;
@@ -546,10 +550,10 @@ int mspr_launch_scores_f32(const void* q, int q_dtype, int n_heads, const float*
   do {                                                                                                  \
     if (stage_half)                                                                                     \
       scores_f32_kernel<DT, true><<<grid, block, 0, st>>>(q, n_heads, pooled, n_rows, weights, scale, scores, kvp, \
-                                                          inv_freq, params, rop);                        \
+                                                          inv_freq, params, rop, valid_rows);            \
     else                                                                                                \
       scores_f32_kernel<DT, false><<<grid, block, 0, st>>>(q, n_heads, pooled, n_rows, weights, scale, scores, kvp, \
-                                                           inv_freq, params, rop);                        \
+                                                           inv_freq, params, rop, valid_rows);            \
   } while (0)
   if (q_dtype == MSPR_F32) MSPR_SCORES_LAUNCH(MSPR_F32);
   else if (q_dtype == MSPR_F16) MSPR_SCORES_LAUNCH(MSPR_F16);
@@ -568,7 +572,7 @@ extern "C" int mspr_fused_qat_indexer_scores(const void* q, int q_dtype, int n_h
   MSPR_REQUIRE(q_dtype >= MSPR_F32 && q_dtype <= MSPR_BF16, "fused_qat_indexer_scores: q must be f32, f16 or bf16");
   MSPR_REQUIRE(mspr_aligned(q, 16) && mspr_aligned(pooled_qat, 16), "fused_qat_indexer_scores: q and pooled_qat must be 16-byte aligned");
   return mspr_launch_scores_f32(q, q_dtype, n_heads, pooled_qat, n_rows, weights, scale, scores, false, nullptr,
-                                nullptr, nullptr, nullptr, (hipStream_t)stream);
+                                nullptr, nullptr, nullptr, nullptr, (hipStream_t)stream);
 }
 
 extern "C" int mspr_indexer_score_tail(const float* scores, int n_heads, int64_t capacity, const void* weights_raw,

@@ -66,6 +66,7 @@ struct SparseAttnArgs {
   const void* pool;
   int64_t pool_batch_stride;
   int64_t n_pool;
+  const int32_t* pool_rows_dev;  // optional: rows of the pool in use, read on the device (<= n_pool, the capacity)
   const int32_t* idx;
   int64_t idx_batch_stride;
   int n_idx;
@@ -418,6 +419,11 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   }
 
   // ---- row pointer and validity of the gathered slots, by all threads at once
+  int64_t n_pool = a.n_pool;
+  if (a.pool_rows_dev) {
+    const int64_t in_use = a.pool_rows_dev[0];
+    n_pool = in_use < n_pool ? (in_use > 0 ? in_use : 0) : n_pool;
+  }
 #pragma unroll
   for (int tj = 0; tj < G::kMaxIds / kThreads; tj++) {
     if (tj * kThreads >= n_tiles * kTile) break;
@@ -429,7 +435,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
       const int id = gi < stop_pos ? my_id[tj] : -1;
       if (id >= 0) {
         const int64_t r = (int64_t)id * a.row_mul + a.row_add;
-        if (r >= 0 && r < a.n_pool) {
+        if (r >= 0 && r < n_pool) {
           valid = true;
           ptr = reinterpret_cast<uint64_t>(pool_b + r * DK);
         }
@@ -952,11 +958,10 @@ extern "C" int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, 
   return run_sparse_attention(a, MSPR_F16, 512, workspace, workspace_bytes_given, (hipStream_t)stream);
 }
 
-extern "C" int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* window, int window_rows,
-                                      const void* row, const void* pooled, int64_t n_rows, const int32_t* sel,
-                                      int n_sel, const void* sinks, const float* inv_freq, const int32_t* params,
-                                      float scale, void* out, void* workspace,
-                                      size_t workspace_bytes_given, void* stream) {
+static int decode_sdpa(const void* q, int n_heads, const void* window, int window_rows, const void* row,
+                       const void* pooled, int64_t n_rows, const int32_t* sel, int n_sel, const void* sinks,
+                       const float* inv_freq, const int32_t* params, float scale, void* out, void* workspace,
+                       size_t workspace_bytes_given, bool fixed, void* stream) {
   MSPR_REQUIRE(q && window && row && pooled && sinks && inv_freq && params && out,
                "fused_decode_sdpa: null pointer");
   MSPR_REQUIRE(n_sel == 0 || sel, "fused_decode_sdpa: null sel");
@@ -994,7 +999,26 @@ extern "C" int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* wi
   a.rope = 1;
   a.out = out;
   a.out_dtype = MSPR_F16;
+  a.pool_rows_dev = fixed ? params + 2 : nullptr;
   return run_sparse_attention(a, MSPR_F16, 512, workspace, workspace_bytes_given, (hipStream_t)stream);
+}
+
+extern "C" int mspr_fused_decode_sdpa(const void* q, int n_heads, const void* window, int window_rows,
+                                      const void* row, const void* pooled, int64_t n_rows, const int32_t* sel,
+                                      int n_sel, const void* sinks, const float* inv_freq, const int32_t* params,
+                                      float scale, void* out, void* workspace, size_t workspace_bytes_given,
+                                      void* stream) {
+  return decode_sdpa(q, n_heads, window, window_rows, row, pooled, n_rows, sel, n_sel, sinks, inv_freq, params, scale,
+                     out, workspace, workspace_bytes_given, false, stream);
+}
+
+extern "C" int mspr_fused_decode_sdpa_fixed(const void* q, int n_heads, const void* window, int window_rows,
+                                            const void* row, const void* pooled, int64_t capacity,
+                                            const int32_t* sel, int n_sel, const void* sinks, const float* inv_freq,
+                                            const int32_t* params, float scale, void* out, void* workspace,
+                                            size_t workspace_bytes_given, void* stream) {
+  return decode_sdpa(q, n_heads, window, window_rows, row, pooled, capacity, sel, n_sel, sinks, inv_freq, params,
+                     scale, out, workspace, workspace_bytes_given, true, stream);
 }
 
 static int sparse_mla_decode_impl(const void* q, const void* kv, const int32_t* rows, const float* sinks, int dtype,

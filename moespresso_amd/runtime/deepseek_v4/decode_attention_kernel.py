@@ -65,8 +65,14 @@ def fp8_kv_prefix_rows(x: torch.Tensor) -> torch.Tensor:
     return out.reshape(x.shape)
 
 
-def fused_decode_prep(q_idx, pooled_qat, weights, kv_row, inv_freq, params, *, scale, topk):
+def fused_decode_prep(q_idx, pooled_qat, weights, kv_row, inv_freq, params, *, scale, topk,
+                      pool_rows_in_params: bool = False):
     """Score, select, and prepare the KV row for one ratio-4 decode token (reference :669).
+
+    With ``pool_rows_in_params`` (an extension for the fixed-capacity decode state, reference
+    fixed_decode_state.py:186-206) ``pooled_qat`` is a capacity buffer and ``params`` is int32
+    ``[position, write_idx, rows in use]``: the row count is read on the device, rows not in use score
+    ``-inf``, so a launch captured in a HIP graph follows the pool as it grows.
 
     Args:
         q_idx: ``[n_heads, 128]`` post-rope, pre-QAT indexer queries (f32/f16/bf16).
@@ -108,6 +114,8 @@ def fused_decode_prep(q_idx, pooled_qat, weights, kv_row, inv_freq, params, *, s
         raise ValueError("inv_freq must be float32 [32]")
     if params.dtype != torch.int32 or params.numel() < 1:
         raise ValueError("params must be int32 with the position at index 0")
+    if pool_rows_in_params and params.numel() < 3:
+        raise ValueError("params must be int32 [position, write_idx, pool_rows] for a fixed-capacity pool")
     dev = _lib.require_device(q_idx, pooled_qat, weights, kv_row, inv_freq, params)
     qc = q_idx.contiguous()
     pc = pooled_qat.contiguous()
@@ -118,7 +126,8 @@ def fused_decode_prep(q_idx, pooled_qat, weights, kv_row, inv_freq, params, *, s
     sel = torch.empty((topk,), dtype=torch.int32, device=dev)
     row = torch.empty((_HEAD_DIM,), dtype=torch.float16, device=dev)
     scores = torch.empty((n_rows,), dtype=torch.float32, device=dev)
-    rc = _lib.lib().mspr_fused_decode_prep(
+    entry = _lib.lib().mspr_fused_decode_prep_fixed if pool_rows_in_params else _lib.lib().mspr_fused_decode_prep
+    rc = entry(
         _lib.ptr(qc), _lib.DTYPE_CODE[q_idx.dtype], n_heads, _lib.ptr(pc), n_rows, _lib.ptr(wc),
         _lib.ptr(kc), _lib.ptr(fc), _lib.ptr(prm), float(scale), topk, _lib.ptr(sel), _lib.ptr(row),
         _lib.ptr(scores), _lib.stream_ptr())
@@ -126,8 +135,12 @@ def fused_decode_prep(q_idx, pooled_qat, weights, kv_row, inv_freq, params, *, s
     return sel, row, scores
 
 
-def fused_decode_sdpa(q, window, row, pooled, sel, sinks, inv_freq, params, *, scale):
+def fused_decode_sdpa(q, window, row, pooled, sel, sinks, inv_freq, params, *, scale,
+                      pool_rows_in_params: bool = False, workspace=None):
     """Attend one decode token over the window and selected pooled rows (reference :733).
+
+    With ``pool_rows_in_params`` ``pooled`` is a capacity buffer and ``params`` is int32 ``[position,
+    write_idx, rows in use]``; ids that name a row not in use are skipped like negative ones.
 
     Args:
         q: float16 ``[n_heads, 512]`` post-norm, pre-rope query heads.
@@ -163,6 +176,8 @@ def fused_decode_sdpa(q, window, row, pooled, sel, sinks, inv_freq, params, *, s
         raise ValueError("inv_freq must be float32 [32]")
     if params.dtype != torch.int32 or params.numel() < 2:
         raise ValueError("params must be int32 [position, write_idx]")
+    if pool_rows_in_params and params.numel() < 3:
+        raise ValueError("params must be int32 [position, write_idx, pool_rows] for a fixed-capacity pool")
     dev = _lib.require_device(q, window, row, pooled, sel, sinks, inv_freq, params)
     window_rows = int(window.shape[0])
     n_rows = int(pooled.shape[0])
@@ -170,8 +185,9 @@ def fused_decode_sdpa(q, window, row, pooled, sel, sinks, inv_freq, params, *, s
     qc, wc, rc_, pc = q.contiguous(), window.contiguous(), row.contiguous(), pooled.contiguous()
     sc, kc, fc, prm = sel.contiguous(), sinks.contiguous(), inv_freq.reshape(-1).contiguous(), params.reshape(-1).contiguous()
     out = torch.empty((n_heads, _HEAD_DIM), dtype=torch.float16, device=dev)
-    ws = _lib.sparse_attention_workspace(1, n_heads, window_rows + n_sel, dev)
-    rc = _lib.lib().mspr_fused_decode_sdpa(
+    ws = workspace if workspace is not None else _lib.sparse_attention_workspace(1, n_heads, window_rows + n_sel, dev)
+    entry = _lib.lib().mspr_fused_decode_sdpa_fixed if pool_rows_in_params else _lib.lib().mspr_fused_decode_sdpa
+    rc = entry(
         _lib.ptr(qc), n_heads, _lib.ptr(wc), window_rows, _lib.ptr(rc_), _lib.ptr(pc), n_rows, _lib.ptr(sc),
         n_sel, _lib.ptr(kc), _lib.ptr(fc), _lib.ptr(prm), float(scale), _lib.ptr(out), _lib.ptr(ws),
         ws.numel() * 4, _lib.stream_ptr())
