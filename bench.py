@@ -329,6 +329,15 @@ def bench_ds4_prefill(dev, gen, reps=5):
     return out
 
 
+def calibration_copy(dev):
+    """One elementwise kernel that reads 1 GiB and writes 1 GiB: the scale of the HBM byte counters."""
+    src = torch.ones(1 << 28, device=dev, dtype=torch.float32)
+    dst = torch.empty_like(src)
+    torch.add(src, 1.0, out=dst)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -341,6 +350,8 @@ def main() -> int:
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one elementwise kernel that reads 1 GiB and writes 1 GiB (scale for HBM counters)")
     ap.add_argument("--headline-only", action="store_true", help="skip the per-config extras")
+    ap.add_argument("--only", default="", help="run just these extras (comma list of prefill, prefill_q8, q8_decode, "
+                                               "ds4_prefill) and print them; for counter runs of one kernel")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every box has one MI355X); rerun with --gpus 1",
@@ -356,6 +367,14 @@ def main() -> int:
 
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev).manual_seed(0)
+    if args.only:
+        legs = {"prefill": bench_prefill, "prefill_q8": bench_prefill_q8, "q8_decode": bench_q8_decode,
+                "ds4_prefill": bench_ds4_prefill}
+        out = {name: legs[name](dev, gen) for name in args.only.split(",")}
+        if args.calibration_copy:
+            calibration_copy(dev)
+        print(json.dumps(out))
+        return 0
     B, R, K, W = args.batch, max(1, args.sets), args.steps, args.warmup
     sets = [make_set(B, dev, gen) for _ in range(R)]
     ws = _lib.sparse_attention_workspace(B, N_HEADS, TOPK + WINDOW, dev)
@@ -485,11 +504,7 @@ def main() -> int:
         "layers_per_graph_replay": R,
     }
     if args.calibration_copy:
-        src = torch.ones(1 << 28, device=dev, dtype=torch.float32)
-        dst = torch.empty_like(src)
-        torch.add(src, 1.0, out=dst)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(dev)
 
     line = {
         "metric": "sparse decode attn us/layer @128K ctx (indexer score + top-2048 + indexed MLA decode)",

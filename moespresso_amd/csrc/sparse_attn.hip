@@ -85,6 +85,7 @@ struct SparseAttnArgs {
   // split: range sp of a sequence owns window slots [sp*win_per_split, +win_per_split) and gathered
   // ids [sp*idx_per_split, +idx_per_split)
   int n_splits;
+  uint32_t inv_splits, inv_hblk, inv_tokens;  // floor(2^32 / n) of n_splits, n_hblk, n_tokens
   int win_per_split;
   int idx_per_split;
   int n_hblk;
@@ -259,11 +260,19 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
   const int total = gridDim.x;
   int work = blockIdx.x;
   if ((total & 7) == 0) work = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
-  const int sp = work % a.n_splits;
-  const int bh = work / a.n_splits;
-  const int hb = bh % a.n_hblk;
-  const int seq = bh / a.n_hblk;
-  const int b = seq / a.n_tokens;
+  // (divisions by multiplication with floor(2^32 / n) and one correction step: a launch starts with an empty
+  // instruction cache, and a software division is a hundred instructions in front of the first memory request)
+  auto div_by = [](uint32_t x, uint32_t n, uint32_t inv) -> uint32_t {
+    if (n == 1u) return x;
+    uint32_t q = __umulhi(x, inv);  // true quotient or one less
+    if (x - q * n >= n) q++;
+    return q;
+  };
+  const int bh = (int)div_by((uint32_t)work, (uint32_t)a.n_splits, a.inv_splits);
+  const int sp = work - bh * a.n_splits;
+  const int seq = (int)div_by((uint32_t)bh, (uint32_t)a.n_hblk, a.inv_hblk);
+  const int hb = bh - seq * a.n_hblk;
+  const int b = (int)div_by((uint32_t)seq, (uint32_t)a.n_tokens, a.inv_tokens);
   const int t = seq - b * a.n_tokens;
 
   // window rows and visible pool prefix of this sequence; the prefill form derives them from the
@@ -383,7 +392,9 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
         if (slot == subst_slot) {
           ptr = reinterpret_cast<uint64_t>(a.subst_row);
         } else {
-          uint32_t r = ((uint32_t)a.raw_start + (uint32_t)seq_win_first + (uint32_t)slot) % (uint32_t)a.raw_cap;
+          // (raw_start and first + slot are both below raw_cap)
+          uint32_t r = (uint32_t)a.raw_start + (uint32_t)seq_win_first + (uint32_t)slot;
+          if (r >= (uint32_t)a.raw_cap) r -= (uint32_t)a.raw_cap;
           ptr = reinterpret_cast<uint64_t>(win_b + (int64_t)r * DK);
         }
       }
@@ -872,6 +883,10 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   const int table_slots = (a.win_per_split + kTile - 1) / kTile * kTile + (a.idx_per_split + kTile - 1) / kTile * kTile;
   MSPR_REQUIRE(table_slots <= 1024, "sparse attention: too many key slots (%d)", n_keys);
   a.direct = a.n_splits == 1;
+  auto magic = [](int n) -> uint32_t { return n <= 1 ? 0u : (uint32_t)(((uint64_t)1 << 32) / (uint32_t)n); };
+  a.inv_splits = magic(a.n_splits);
+  a.inv_hblk = magic(a.n_hblk);
+  a.inv_tokens = magic(a.n_tokens);
   size_t need = workspace_bytes(a.batch, a.n_heads, n_keys);
   MSPR_REQUIRE(workspace && workspace_bytes_given >= need, "sparse attention: workspace of %zu bytes needed, %zu given",
                need, workspace_bytes_given);
