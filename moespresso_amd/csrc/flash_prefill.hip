@@ -135,7 +135,7 @@ __device__ __forceinline__ int swz(int r) { return ((r & 7) << 1) | ((r >> 3) & 
 
 // Q8 = false: k / v are the whole 16-bit cache, q / out have its element type.
 // Q8 = true (KDT float16): float32 q / out, quantised prefix + float16 tail rows (see PrefillArgs).
-template <int KDT, bool Q8, int SDT>
+template <int KDT, bool Q8, int SDT, bool IO32 = Q8>
 __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs a) {
   extern __shared__ __attribute__((aligned(256))) unsigned char lds[];  // tile bases: zero low bits under the address XORs
   const int tid = threadIdx.x;
@@ -217,7 +217,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
     if (qrow > a.q_len - 1) qrow = a.q_len - 1;
     if (qrow < 0) qrow = 0;
     const int64_t qoff = (((int64_t)b * a.n_q_heads + head) * a.q_len + qrow) * kD + 8 * g;
-    if constexpr (!Q8) {
+    if constexpr (!IO32) {
       const u32x4_t* qp = reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint16_t*>(a.q) + qoff);
 #pragma unroll
       for (int s = 0; s < 16; s++) qf[s] = qp[2 * s];
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
     for (int mt = 0; mt < 8; mt++)
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        if constexpr (Q8) {
+        if constexpr (IO32) {
           *reinterpret_cast<f32x4_t*>(reinterpret_cast<float*>(a.out) + ooff + 32 * mt + 8 * c + 4 * g) =
               f32x4_t{oacc[mt][4 * c] * inv, oacc[mt][4 * c + 1] * inv, oacc[mt][4 * c + 2] * inv,
                       oacc[mt][4 * c + 3] * inv};
@@ -525,9 +525,9 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
 template <int SDT>
 __global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, const void* self_k, const void* self_v,
                                                               int self_dtype, uint16_t* tail_k, uint16_t* tail_v,
-                                                              int tail_rows) {
+                                                              int tail_rows, int first_row) {
   const int d = threadIdx.x;
-  const int j = blockIdx.x;
+  const int j = first_row + blockIdx.x;
   const int kvh = blockIdx.y;
   const int b = blockIdx.z;
   const int64_t bh = (int64_t)b * a.n_kv_heads + kvh;
@@ -558,6 +558,37 @@ __global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, con
   vx = __builtin_amdgcn_fmed3f(vx, -65504.0f, 65504.0f);
   tail_k[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(kx);
   tail_v[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(vx);
+}
+
+// Prefix rows [0, n_rows) of the quantised cache as float16 rows of the dense K/V buffers (the form taken for
+// long chunks: the attention kernel then reads every tile as a dense one). Same arithmetic as the in-kernel
+// unpacking (float16 code * scale + bias), so both forms attend the same values. A thread converts 16 codes
+// of K and of V; 16 threads a row, 16 rows a workgroup.
+template <int SDT>
+__global__ __launch_bounds__(256) void prefill_q8_dequant_kernel(PrefillArgs a, uint16_t* out_k, uint16_t* out_v,
+                                                                 int64_t n_rows, int64_t out_rows) {
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+  const int pp = threadIdx.x & 15;
+  if (row >= n_rows) return;
+  const int64_t bh = (int64_t)blockIdx.z * a.n_kv_heads + blockIdx.y;
+  const int64_t src = bh * a.past_rows + row;
+  const u32x4_t rk = reinterpret_cast<const u32x4_t*>(a.pk_wq)[src * 16 + pp];
+  const u32x4_t rv = reinterpret_cast<const u32x4_t*>(a.pv_wq)[src * 16 + pp];
+  uint32_t rs[4];
+  const void* arrs[4] = {a.pk_s, a.pk_b, a.pv_s, a.pv_b};
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    if constexpr (SDT == MSPR_F32) rs[i] = reinterpret_cast<const uint32_t*>(arrs[i])[src * 4 + (pp >> 2)];
+    else rs[i] = reinterpret_cast<const uint16_t*>(arrs[i])[src * 4 + (pp >> 2)];
+  }
+  u32x4_t p0, p1;
+  const int64_t dst = (bh * out_rows + row) * kD + 16 * pp;
+  dequant16(rk, sb_to_h2<SDT>(rs[0]), sb_to_h2<SDT>(rs[1]), p0, p1);
+  *reinterpret_cast<u32x4_t*>(out_k + dst) = p0;
+  *reinterpret_cast<u32x4_t*>(out_k + dst + 8) = p1;
+  dequant16(rv, sb_to_h2<SDT>(rs[2]), sb_to_h2<SDT>(rs[3]), p0, p1);
+  *reinterpret_cast<u32x4_t*>(out_v + dst) = p0;
+  *reinterpret_cast<u32x4_t*>(out_v + dst + 8) = p1;
 }
 
 // Merge of the key-range partials of one query row: 64 lanes x 4 columns, four rows per workgroup.
@@ -641,11 +672,11 @@ size_t prefill_split_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len, 
   return (size_t)splits * batch * n_q_heads * q_len * (kD + 2) * sizeof(float);
 }
 
-template <int KDT, bool Q8, int SDT>
+template <int KDT, bool Q8, int SDT, bool IO32 = Q8>
 int prefill_launch(const PrefillArgs& a, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&flash_prefill_kernel<KDT, Q8, SDT>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&flash_prefill_kernel<KDT, Q8, SDT, IO32>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     if (e != hipSuccess) {
       mspr_set_error("flash_prefill: cannot reserve %d bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
@@ -656,13 +687,13 @@ int prefill_launch(const PrefillArgs& a, hipStream_t st) {
   dim3 grid((unsigned)(a.q_blocks * a.n_kv_heads * a.batch * a.n_splits)), block(kThreads);
   {
     MsprProfScope prof(MSPR_K_FLASH_PREFILL, st);
-    flash_prefill_kernel<KDT, Q8, SDT><<<grid, block, kLdsBytes, st>>>(a);
+    flash_prefill_kernel<KDT, Q8, SDT, IO32><<<grid, block, kLdsBytes, st>>>(a);
   }
   MSPR_CHECK_LAUNCH("flash_prefill");
   if (a.n_splits > 1) {
     const int64_t n_rows = (int64_t)a.batch * a.n_q_heads * a.q_len;
     dim3 mgrid((unsigned)((n_rows + 3) / 4)), mblock(256);
-    if (Q8) prefill_merge_kernel<MSPR_F32><<<mgrid, mblock, 0, st>>>(a);
+    if (IO32) prefill_merge_kernel<MSPR_F32><<<mgrid, mblock, 0, st>>>(a);
     else prefill_merge_kernel<KDT><<<mgrid, mblock, 0, st>>>(a);
     MSPR_CHECK_LAUNCH("flash_prefill (merge)");
   }
@@ -722,12 +753,18 @@ extern "C" int mspr_flash_prefill(const void* q, const void* k, const void* v, i
   return prefill_launch<MSPR_F16, false, MSPR_F32>(a, st);
 }
 
+// Prefix tiles unpacked inside the attention kernel. Unpacking costs a fifth of a tile's time for every
+// workgroup that passes the tile; converting the prefix once costs about 1.4 ns per row. From a thousand
+// queries per chunk on, the prefix is therefore converted to float16 rows first (a scratch of 1 KB per key and
+// KV head) and the attention kernel runs on dense tiles only.
+static int prefill_q8_tiles(int q_len, int64_t past_len) { return q_len >= 1024 ? 0 : (int)(past_len / kTile); }
+
 extern "C" size_t mspr_sdpa_fa_prefill_q8_workspace_bytes(int batch, int n_q_heads, int n_kv_heads, int q_len,
                                                           int64_t past_len) {
   if (batch < 1 || n_kv_heads < 1 || n_q_heads < n_kv_heads || n_q_heads % n_kv_heads != 0 || q_len < 1 ||
       past_len < 0 || n_q_heads / n_kv_heads > 8)
     return 0;
-  const int64_t tail_rows = past_len % kTile + q_len;
+  const int64_t tail_rows = past_len - (int64_t)prefill_q8_tiles(q_len, past_len) * kTile + q_len;
   const size_t tail = ((size_t)batch * n_kv_heads * tail_rows * kRowBytes * 2 + 255) / 256 * 256;
   return tail + prefill_split_bytes(batch, n_q_heads, n_kv_heads, q_len, past_len) + 256;
 }
@@ -763,7 +800,8 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
   MSPR_REQUIRE(workspace && workspace_bytes >= need && mspr_aligned(workspace, 16),
                "sdpa_fa_prefill_q8: workspace of %zu bytes (16-byte aligned) needed, %zu given", need, workspace_bytes);
   PrefillArgs a = {};
-  const int tail_rows = (int)(past_len % kTile) + q_len;
+  const int q8_tiles = prefill_q8_tiles(q_len, past_len);
+  const int tail_rows = (int)(past_len - (int64_t)q8_tiles * kTile) + q_len;
   uint16_t* tail_k = reinterpret_cast<uint16_t*>(workspace);
   uint16_t* tail_v = tail_k + (size_t)batch * n_kv_heads * tail_rows * kD;
   a.q = queries;
@@ -779,7 +817,7 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
   a.scale_log2 = (float)((double)scale * 1.4426950408889634);
   a.rep_shift = rep == 1 ? 0 : rep == 2 ? 1 : rep == 4 ? 2 : 3;
   a.q_blocks = prefill_q_blocks(rep, q_len);
-  a.q8_tiles = (int)(past_len / kTile);
+  a.q8_tiles = q8_tiles;
   a.past_rows = past_rows;
   a.n_splits = prefill_choose_splits(batch, n_kv_heads, a.q_blocks, past_len, q_len);
   if (a.n_splits > 1) {
@@ -794,11 +832,23 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
   a.pv_s = pv_scales;
   a.pv_b = pv_biases;
   hipStream_t st = (hipStream_t)stream;
-  dim3 tgrid((unsigned)tail_rows, (unsigned)n_kv_heads, (unsigned)batch);
-  if (sb_dtype == MSPR_F32) prefill_q8_tail_kernel<MSPR_F32><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows);
-  else if (sb_dtype == MSPR_F16) prefill_q8_tail_kernel<MSPR_F16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows);
-  else prefill_q8_tail_kernel<MSPR_BF16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows);
+  // rows of the dense buffers: prefix rows not left to the attention kernel, then the chunk's own rows
+  const int64_t dq_rows = q8_tiles == 0 ? past_len : 0;  // converted 16 codes at a time
+  const int first_row = (int)dq_rows;                   // the rest element by element (at most 31 prefix rows + chunk)
+  if (dq_rows > 0) {
+    dim3 dgrid((unsigned)((dq_rows + 15) / 16), (unsigned)n_kv_heads, (unsigned)batch);
+    if (sb_dtype == MSPR_F32) prefill_q8_dequant_kernel<MSPR_F32><<<dgrid, 256, 0, st>>>(a, tail_k, tail_v, dq_rows, tail_rows);
+    else if (sb_dtype == MSPR_F16) prefill_q8_dequant_kernel<MSPR_F16><<<dgrid, 256, 0, st>>>(a, tail_k, tail_v, dq_rows, tail_rows);
+    else prefill_q8_dequant_kernel<MSPR_BF16><<<dgrid, 256, 0, st>>>(a, tail_k, tail_v, dq_rows, tail_rows);
+    MSPR_CHECK_LAUNCH("sdpa_fa_prefill_q8 (prefix rows)");
+  }
+  dim3 tgrid((unsigned)(tail_rows - first_row), (unsigned)n_kv_heads, (unsigned)batch);
+  if (sb_dtype == MSPR_F32) prefill_q8_tail_kernel<MSPR_F32><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows, first_row);
+  else if (sb_dtype == MSPR_F16) prefill_q8_tail_kernel<MSPR_F16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows, first_row);
+  else prefill_q8_tail_kernel<MSPR_BF16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows, first_row);
   MSPR_CHECK_LAUNCH("sdpa_fa_prefill_q8 (tail rows)");
+  // (prefix converted beforehand: the dense kernel, with float32 queries and output)
+  if (q8_tiles == 0) return prefill_launch<MSPR_F16, false, MSPR_F32, true>(a, st);
   if (sb_dtype == MSPR_F32) return prefill_launch<MSPR_F16, true, MSPR_F32>(a, st);
   if (sb_dtype == MSPR_F16) return prefill_launch<MSPR_F16, true, MSPR_F16>(a, st);
   return prefill_launch<MSPR_F16, true, MSPR_BF16>(a, st);

@@ -130,6 +130,8 @@ def _q8_inputs(past, L, seed, sb_dtype=torch.float32, Hq=16, Hkv=2, B=1):
     (31, 1, torch.float32, torch.float32),
     (4133, 40, torch.float32, torch.float32),   # key-range splits over the quantised prefix
     (6000, 256, torch.bfloat16, torch.float32),
+    (700, 1100, torch.bfloat16, torch.float32),   # long chunk: the prefix is converted to float16 rows first
+    (45, 1024, torch.float32, torch.bfloat16),
 ])
 def test_sdpa_fa_prefill_q8_matches_oracle(past, L, sb_dtype, self_dtype):
     """Tolerance 1e-2 max-abs (8-bit KV bar) vs float64 attention over the dequantised prefix + chunk."""
