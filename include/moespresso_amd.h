@@ -312,7 +312,9 @@ int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, const void* 
  * k with HIP events on the launch stream (0 switches it off; it must be off under stream capture).
  * Kernel ids: 1 fp8 indexer scores, 2 top-k, 3 sparse attention split, 4 sparse attention merge,
  * 5 float32 indexer scores, 6 Q8 decode split, 7 Q8 decode merge, 8 flash prefill.
- * No counterpart in the reference (its probes time whole calls on the host). */
+ * No counterpart in the reference (its probes time whole calls on the host). These two are the
+ * exception to "never allocates, never synchronises": enabling makes the launchers create HIP events
+ * (kept and reused), and mspr_profile_collect waits for the recorded launches. */
 int mspr_profile_enable(int kernel_mask);
 
 /* Waits for the recorded launches of kernel_id, writes their durations in milliseconds to the HOST

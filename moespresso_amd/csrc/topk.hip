@@ -19,22 +19,6 @@
 #include "common.h"
 #include "profile.h"
 
-#ifdef MSPR_TOPK_TRACE
-// Debug build only: cycle stamps of the phases of workgroup 0.
-__device__ long long g_topk_trace[32];
-extern "C" int mspr_debug_topk_trace(long long* host_out) {
-  return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_topk_trace), sizeof(long long) * 32);
-}
-#define TOPK_STAMP(i)                                                      \
-  do {                                                                     \
-    if (blockIdx.x == 0 && threadIdx.x == 0) g_topk_trace[i] = clock64(); \
-  } while (0)
-#else
-#define TOPK_STAMP(i) \
-  do {                \
-  } while (0)
-#endif
-
 namespace {
 
 constexpr int kThreads = 1024;
@@ -423,7 +407,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
   if (sample_rank > 0)
     for (int i = tid; i < 5 * 256; i += kThreads) (&fhist[0][0])[i] = 0u;  // ordered by the barriers of the load
 
-  TOPK_STAMP(0);
   // Load with lane-contiguous 16-byte reads (a wave reads 1 KB at a time), then hand every thread its
   // C consecutive rows through LDS. The 16-byte pieces of a thread's C/4-piece block are XOR-permuted
   // by the thread index so that neither the writes nor the reads pile up on a few banks.
@@ -464,7 +447,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
       for (int e = 0; e < 4; e++) kreg[4 * j + e] = keys[e];
     }
   }
-  TOPK_STAMP(1);
 
   // ---- pivot path. Every thread's first row is a sample of the (padded) row set; the 16-bit key
   // prefix at rank `sample_rank` of the sample sits, with a wide margin, below the k-th key of the
@@ -494,7 +476,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
     const Pick s1 = shared_pick(fhist[1], s0.need, 1);
     const uint32_t pivot16 = (s0.digit << 8) | s1.digit;
     const uint32_t pivot = pivot16 << 16;
-    TOPK_STAMP(2);
 
     uint32_t smask = 0u;
 #pragma unroll
@@ -510,7 +491,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
       sbase += w < wave ? wt : 0u;
       total += wt;
     }
-    TOPK_STAMP(3);
     if (total >= (uint32_t)topk && total <= (uint32_t)kFastCap) {  // the same for every thread
       uint32_t pos = sbase + sincl - cnt;
       while (smask) {
@@ -519,7 +499,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
         fast_rows[pos++] = (uint16_t)(C * tid + i);
       }
       __syncthreads();
-      TOPK_STAMP(4);
       // thread t takes the list entries [t E, t E + E): consecutive, so the emission order is again a
       // matter of one block scan
       const uint32_t per = (total + kThreads - 1) / kThreads;  // 1 .. kFastPer
@@ -560,7 +539,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
           fprefix |= pk.digit << shift;
           fneed = pk.need;
         }
-        TOPK_STAMP(14);
         const uint32_t n_above_f = (uint32_t)topk - fneed;
         uint32_t am = 0u, tm = 0u;
 #pragma unroll
@@ -583,7 +561,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
           if ((am >> j) & 1u) sel[slot_f++] = (int32_t)lr[j];
           else if (((tm >> j) & 1u) && rank_f < fneed) sel[n_above_f + rank_f++] = (int32_t)lr[j];
         }
-        TOPK_STAMP(17);
         return;
       }
     }
@@ -609,9 +586,7 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
       const uint32_t key = kreg[i];
       if (pass == 0 || (key & mask_hi) == prefix) atomicAdd(&hist[((key >> shift) & 0xFFu) * kCopies + lane], 1u);
     }
-    TOPK_STAMP(2 + 3 * pass);
     __syncthreads();
-    TOPK_STAMP(3 + 3 * pass);
     // totals[bin] = sum over copies: four threads per bin, 16 copies each as four 16-byte reads
     // (rotated so that 16 neighbouring lanes cover all 16 bank groups), zeroed behind the read
     {
@@ -633,7 +608,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
     prefix |= p.digit << shift;
     need = p.need;
     live = p.live;
-    TOPK_STAMP(4 + 3 * pass);
   };
 
   full_pass(0);
@@ -671,7 +645,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
   const uint32_t threshold = prefix;
   const uint32_t need_ties = need;
   const uint32_t n_above = (uint32_t)topk - need_ties;
-  TOPK_STAMP(14);
 
   // ---- ordered emission: per-thread masks, one packed block scan (above count low, tie count high)
   uint32_t above_mask = 0u, tie_mask = 0u;
@@ -683,9 +656,7 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
   const uint32_t mine = (uint32_t)__popc(above_mask) | ((uint32_t)__popc(tie_mask) << 16);
   const uint32_t incl = wave_prefix_sum(mine);
   if (lane == 63) wave_tot[wave] = incl;
-  TOPK_STAMP(15);
   __syncthreads();
-  TOPK_STAMP(16);
   uint32_t base = 0u;
   for (int w = 0; w < wave; w++) base += wave_tot[w];
   const uint32_t excl = base + incl - mine;
@@ -702,7 +673,6 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
     tie_mask &= tie_mask - 1u;
     sel[n_above + rank_t++] = row0 + i;
   }
-  TOPK_STAMP(17);
 }
 
 // Rank, inside the 1024-row sample, of the pivot of the pivot path; 0 switches the path off. With k of
