@@ -724,6 +724,493 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 }
 
 // Merge of the per-split partials: one workgroup per (batch, head block, wave slot, 32-column tile).
+// ---------------------------------------------------------------------------------------------------
+// Prefill consumer: many query tokens against one ring of raw rows and one pool (float16 rows of 512).
+//
+// A workgroup is persistent: it takes every gridDim.x-th (token, head block) unit and runs their 32-slot
+// tiles as one stream through the ring of three tile buffers, so that the first rows of the next token are
+// requested while the last tiles of the current one are multiplied. What a token needs before its first
+// tile (ids -> stop position -> row pointers; its query rows) is produced inside the tile loop of the token
+// before it: ids are requested at tile 0, the row pointer table is written at tile 1 into the other of
+// two table slots, the query operand is requested behind the last S^T product. Every token runs at least
+// kMinTiles tiles (the missing ones are fully masked), which is what makes those positions exist.
+//
+// The tile step differs from the split kernel's. The four waves of a head group still contract a quarter
+// of the row width each, but a wave then sums only a quarter of the keys (8 of the 32: registers 4 dh ..
+// 4 dh + 3 of the four partial S^T), takes the exponentials of those alone, and writes them as P^T in the
+// element type; every wave reads the 32 x 32 P^T block of its head group back as the B operand of
+// O^T += V^T . P^T. A quarter of the exponentials and of the exchange traffic per wave, at the price of
+// a second barrier. The running maximum has to be the same in the four waves: a wave uses the common
+// m_run as it is, and raises a flag if one of its keys exceeds it by more than kGrow; on a flagged tile
+// (always the first one of a token, rarely another) the four waves exchange their maxima, rescale, and
+// write P^T again.
+//
+// Barriers of step s: B (partial S^T written; every wave has left the V^T reads of step s-1, so the
+// copies of tile s+2 may overwrite its buffer and are issued right behind B) and C (P^T written; every
+// wave has waited for its own copies of tile s+1 before C, so tile s+1 is complete when step s+1 starts).
+// ---------------------------------------------------------------------------------------------------
+struct PrefillGeometry {
+  using G = Geometry<512>;
+  static constexpr int kMaxTiles = 22;                    // 704 slots per token
+  static constexpr int kMinTiles = 4;
+  static constexpr int kTableSlots = kMaxTiles * kTile;
+  static constexpr int kPPitch = 80;                      // bytes per head of P^T: 32 keys + 16 B, so that the
+                                                          // 16 heads of a read phase start on distinct banks
+  static constexpr int kOffSx = G::kBufs * G::kTileBytes;            // [8 waves][4 key octets][64 lanes][4] float
+  static constexpr int kOffTable = kOffSx + kWaves * 4096;           // [2][kTableSlots] row pointers
+  static constexpr int kOffVmask = kOffTable + 2 * kTableSlots * 8;  // [2][32] validity word per tile
+  static constexpr int kOffP = kOffVmask + 2 * 32 * 4;               // [2 head groups][32 heads][kPPitch]
+  static constexpr int kOffTmax = kOffP + 2 * 32 * kPPitch;          // [8 waves][32 heads] float
+  static constexpr int kOffL = kOffTmax + kWaves * 32 * 4;           // [8 waves][32 heads] float
+  static constexpr int kOffFlag = kOffL + kWaves * 32 * 4;           // flag[2], stop[2]
+  static constexpr int kLdsBytes = kOffFlag + 16;
+  static_assert(kOffTable % 16 == 0 && kOffP % 16 == 0 && kLdsBytes <= 160 * 1024, "LDS map of the prefill consumer");
+};
+
+// s_waitcnt vmcnt(n) for a wave-uniform n (the encodable counts that the prefill kernel needs), then the
+// LDS wait and the barrier
+__device__ __forceinline__ void wait_vm_dyn_and_barrier(int n) {
+  switch (n) {
+    case 2: wait_vm_and_barrier<2>(); break;
+    case 4: wait_vm_and_barrier<4>(); break;
+    case 5: wait_vm_and_barrier<5>(); break;
+    case 6: wait_vm_and_barrier<6>(); break;
+    case 7: wait_vm_and_barrier<7>(); break;
+    case 8: wait_vm_and_barrier<8>(); break;
+    case 12: wait_vm_and_barrier<12>(); break;
+    case 13: wait_vm_and_barrier<13>(); break;
+    default: wait_vm_and_barrier<0>(); break;
+  }
+}
+
+struct PrefillUnit {
+  int b, t, hb, seq;
+  int n_win, win_first, wt;  // ring rows of the token's window, first of them (logical), their tiles
+  int64_t visible;
+};
+
+__global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(SparseAttnArgs a) {
+  constexpr int KDT = MSPR_F16;
+  constexpr int DK = 512;
+  using G = Geometry<DK>;
+  using PG = PrefillGeometry;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  unsigned char* kbuf = lds;
+  float* sx = reinterpret_cast<float*>(lds + PG::kOffSx);
+  uint64_t* table = reinterpret_cast<uint64_t*>(lds + PG::kOffTable);
+  uint32_t* vmask = reinterpret_cast<uint32_t*>(lds + PG::kOffVmask);
+  float* tmaxbuf = reinterpret_cast<float*>(lds + PG::kOffTmax);
+  float* lbuf = reinterpret_cast<float*>(lds + PG::kOffL);
+  int* flag = reinterpret_cast<int*>(lds + PG::kOffFlag);
+  int* stop_sh = flag + 2;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int hg = wave >> 2;
+  const int dh = wave & 3;
+  const int n = lane & 31;
+  const int g = lane >> 5;
+  unsigned char* pbuf = lds + PG::kOffP + hg * (32 * PG::kPPitch) + n * PG::kPPitch;
+  const int k_mine = wave < G::kLastWaves ? G::kPerThread : G::kPerThread - 1;  // copies of this wave per tile
+
+  const int n_units = a.batch * a.n_hblk;
+  const int stride = (int)gridDim.x;
+  int unit = (int)blockIdx.x;
+  if (unit >= n_units) return;
+
+  auto div_by = [](uint32_t x, uint32_t n, uint32_t inv) -> uint32_t {
+    if (n == 1u) return x;
+    uint32_t q = __umulhi(x, inv);
+    if (x - q * n >= n) q++;
+    return q;
+  };
+  auto unit_of = [&](int u) -> PrefillUnit {
+    PrefillUnit m;
+    m.seq = (int)div_by((uint32_t)u, (uint32_t)a.n_hblk, a.inv_hblk);
+    m.hb = u - m.seq * a.n_hblk;
+    m.b = (int)div_by((uint32_t)m.seq, (uint32_t)a.n_tokens, a.inv_tokens);
+    m.t = m.seq - m.b * a.n_tokens;
+    // window rows and visible pool prefix, in the unsigned 32-bit arithmetic of the reference kernel
+    const uint32_t qpos = a.pos0 + (uint32_t)m.t, n_raw = (uint32_t)a.raw_cap;
+    const uint32_t last_pos = a.pos0 + (uint32_t)a.n_tokens - 1u;
+    const uint32_t first_raw_pos = last_pos + 1u - n_raw;
+    const uint32_t window_first = (a.window != 0u && qpos + 1u > a.window) ? qpos + 1u - a.window : 0u;
+    const uint32_t first = first_raw_pos > window_first ? first_raw_pos : window_first;
+    const uint32_t last = qpos < last_pos ? qpos : last_pos;
+    m.n_win = first <= last ? (int)(last - first + 1u) : 0;
+    if (m.n_win > a.n_win) m.n_win = a.n_win;
+    m.win_first = first <= last ? (int)(first - first_raw_pos) : 0;
+    const int64_t vis = a.ratio == 0u ? a.n_pool : (int64_t)((qpos + 1u) / a.ratio);
+    m.visible = vis < a.n_pool ? vis : a.n_pool;
+    m.wt = (m.n_win + kTile - 1) / kTile;
+    return m;
+  };
+  auto tiles_of = [&](const PrefillUnit& m, int stop_pos) -> int {
+    const int nt = m.wt + (stop_pos + kTile - 1) / kTile;
+    return nt < PG::kMinTiles ? PG::kMinTiles : nt;
+  };
+  // ids of this thread's two table slots (slot ls = tid + 512 j; gathered part starts at slot 32 wt): always two
+  // loads with every lane active, index clamped, so that the count of loads in flight is the same in every wave
+  auto request_ids = [&](const PrefillUnit& m, int (&ids)[2]) {
+    const int32_t* idx_b = a.idx + (int64_t)m.seq * a.idx_batch_stride;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      int gi = tid + kThreads * j - m.wt * kTile;
+      gi = gi < 0 ? 0 : (gi >= a.n_idx ? a.n_idx - 1 : gi);
+      const int32_t* p = idx_b + gi;
+      asm volatile("global_load_dword %0, %1, off" : "=&v"(ids[j]) : "v"(p) : "memory");
+    }
+  };
+  // position of the first id that ends the walk (>= the visible prefix), minimum over the workgroup
+  auto scan_stop = [&](const PrefillUnit& m, const int (&ids)[2], int* stop) {
+    int first = a.n_idx;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int gi = tid + kThreads * j - m.wt * kTile;
+      if (gi >= 0 && gi < a.n_idx && ids[j] >= 0 && (int64_t)ids[j] >= m.visible && gi < first) first = gi;
+    }
+    if (first < a.n_idx) atomicMin(stop, first);
+  };
+  const uint64_t zero_row = reinterpret_cast<uint64_t>(&g_zero_row[0]);
+  auto build_table = [&](const PrefillUnit& m, int slot, const int (&ids)[2], int stop_pos, int n_tiles) {
+    const uint16_t* win_b = reinterpret_cast<const uint16_t*>(a.win) + (int64_t)m.b * a.win_batch_stride;
+    const uint16_t* pool_b = reinterpret_cast<const uint16_t*>(a.pool) + (int64_t)m.b * a.pool_batch_stride;
+    const int g_ls0 = m.wt * kTile;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int ls = tid + kThreads * j;
+      uint64_t ptr = zero_row;
+      bool valid = false;
+      if (ls < g_ls0) {
+        if (ls < m.n_win) {
+          uint32_t r = (uint32_t)a.raw_start + (uint32_t)m.win_first + (uint32_t)ls;
+          if (r >= (uint32_t)a.raw_cap) r -= (uint32_t)a.raw_cap;
+          valid = true;
+          ptr = reinterpret_cast<uint64_t>(win_b + (int64_t)r * DK);
+        }
+      } else {
+        const int gi = ls - g_ls0;
+        const int id = gi < stop_pos ? ids[j] : -1;
+        if (id >= 0) {
+          const int64_t r = (int64_t)id * a.row_mul + a.row_add;
+          if (r >= 0 && r < a.n_pool) {
+            valid = true;
+            ptr = reinterpret_cast<uint64_t>(pool_b + r * DK);
+          }
+        }
+      }
+      const uint64_t bal = __ballot(valid);
+      if (ls < n_tiles * kTile) {  // (a multiple of 32: whole or half waves)
+        table[slot * PG::kTableSlots + ls] = ptr;
+        if ((lane & 31) == 0) vmask[slot * 32 + (ls >> 5)] = (uint32_t)(bal >> (lane & 32));
+      }
+    }
+  };
+
+  // ---- tile copies (as in the split kernel): LDS slot P = tid + 512 j holds (row P / kSlots, chunk P % kSlots)
+  uint32_t pk[G::kPerThread];
+#pragma unroll
+  for (int j = 0; j < G::kPerThread; j++) {
+    const int P = tid + kThreads * j;
+    const int row = P / G::kSlots, chunk = P % G::kSlots;
+    pk[j] = (P < G::kTileSlots && chunk != G::kSlots - 1) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
+  }
+  auto tile_sources = [&](int slot, int tile, uint64_t (&src)[G::kPerThread]) {
+    const uint64_t* rp = table + slot * PG::kTableSlots + tile * kTile;
+#pragma unroll
+    for (int j = 0; j < G::kPerThread; j++) {
+      const uint32_t p = pk[j];
+      const bool act = p != 0xFFFFFFFFu;
+      src[j] = rp[act ? (p >> 16) : 0] + (act ? (p & 0xFFFFu) : 0u);
+    }
+  };
+  auto tile_lds_base = [&](int buf) -> uint32_t {
+    return __builtin_amdgcn_readfirstlane(
+        (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, kbuf + buf * G::kTileBytes + wave * 1024));
+  };
+  auto issue_copies = [&](const uint64_t (&src)[G::kPerThread], uint32_t dst_lds) {
+#pragma unroll
+    for (int j = 0; j < G::kPerThread; j++)
+      if (j < G::kPerThread - 1 || wave < G::kLastWaves) async_load_16(src[j], dst_lds + j * (kWaves * 1024));
+  };
+
+  // ---- query operand of a unit: lane (n = head, g) holds q[head][dh*128 + 16 ks + 8 g .. +7]
+  u32x4_t qf[G::kSteps];
+  auto request_q = [&](const PrefillUnit& m) {
+    const int head = m.hb * 64 + hg * 32 + n;
+    const int64_t qoff = (int64_t)m.b * a.q_batch_stride + (int64_t)m.t * a.q_token_stride +
+                         (int64_t)(head < a.n_heads ? head : 0) * a.q_head_stride + dh * G::kPart + 8 * g;
+    const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
+#pragma unroll
+    for (int ks = 0; ks < G::kSteps; ks++) {
+      const uint16_t* p = qp + 16 * ks;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(qf[ks]) : "v"(p) : "memory");
+    }
+  };
+  static_assert(G::kSteps == 8, "the query wait below names eight registers");
+  auto await_q = [&](int newer) {  // at most `newer` younger loads of this wave may stay in flight
+    if (newer == G::kPerThread)
+      asm volatile("s_waitcnt vmcnt(%8)" : "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]),
+                   "+v"(qf[6]), "+v"(qf[7]) : "n"(G::kPerThread) : "memory");
+    else if (newer == G::kPerThread - 1)
+      asm volatile("s_waitcnt vmcnt(%8)" : "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]),
+                   "+v"(qf[6]), "+v"(qf[7]) : "n"(G::kPerThread - 1) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]),
+                   "+v"(qf[6]), "+v"(qf[7]) : : "memory");
+  };
+  auto mask_q = [&](const PrefillUnit& m) {
+    if (m.hb * 64 + hg * 32 + n >= a.n_heads) {
+#pragma unroll
+      for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+  };
+
+  // ---- first unit: ids, stop position, table, query, first two tiles
+  PrefillUnit cur = unit_of(unit);
+  int ids[2];
+  const bool have_ids = a.n_idx > 0;
+  if (have_ids) request_ids(cur, ids); else ids[0] = ids[1] = -1;
+  request_q(cur);
+  if (tid == 0) stop_sh[0] = a.n_idx;
+  __syncthreads();
+  if (have_ids) {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(ids[0]), "+v"(ids[1]) : "n"(G::kSteps) : "memory");
+    scan_stop(cur, ids, &stop_sh[0]);
+  }
+  __syncthreads();
+  int n_cur = tiles_of(cur, stop_sh[0]);
+  build_table(cur, 0, ids, stop_sh[0], n_cur);
+  await_q(0);
+  mask_q(cur);
+  // sink of this lane's head (a plain load: its wait would drain the tile copies anywhere behind this point)
+  float sink_l2;
+  {
+    const int head = cur.hb * 64 + hg * 32 + n;
+    sink_l2 = head < a.n_heads ? load_sink_log2(a, head) : -__builtin_inff();
+    asm volatile("" : "+v"(sink_l2));
+  }
+  __syncthreads();
+  {
+    uint64_t src[G::kPerThread];
+    tile_sources(0, 0, src);
+    issue_copies(src, tile_lds_base(0));
+    tile_sources(0, 1, src);
+    issue_copies(src, tile_lds_base(1));
+  }
+
+  f32x16_t oacc[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; mt++) oacc[mt] = f32x16_t{0};
+  float m_run = -__builtin_inff();  // reference maximum per head, the same in the four waves of a head group
+  float l_run = 0.0f;               // this wave's keys only
+
+  const int a_row_off = n * G::kPitch + (dh * G::kPart + 8 * g) * 2;
+  const int tr_s = lane & 15;
+  const int tr_off = (4 * g + (tr_s >> 2)) * G::kPitch + (dh * 128 + 16 * ((lane >> 4) & 1) + 4 * (tr_s & 3)) * 2;
+  constexpr float kGrow = 8.0f;  // float16 weights stay below 2^15
+
+  // tile 0 is complete once every wave's copies of it are (the copies of tile 1 stay in flight)
+  wait_vm_dyn_and_barrier(k_mine);
+
+  int s = 0;    // tiles done by this workgroup: ring buffer s % 3, flag slot s & 1
+  int slot = 0; // table slot of the current unit
+  for (;;) {
+    const bool have_next = unit + stride < n_units;
+    PrefillUnit nxt = cur;
+    int n_nxt = 0;
+    int nids[2] = {-1, -1};
+    if (have_next) nxt = unit_of(unit + stride);
+
+    for (int t = 0; t < n_cur; t++, s++) {
+      const unsigned char* kt = kbuf + (s % G::kBufs) * G::kTileBytes;
+      const bool last = t == n_cur - 1;
+      // ---- S^T partial over this wave's quarter of the row width (two chains of dependent MFMAs)
+      f32x16_t sacc = {0};
+      {
+        f32x16_t sodd = {0};
+        constexpr int kAhead = 6;
+        u32x4_t af[kAhead];
+#pragma unroll
+        for (int ks = 0; ks < kAhead; ks++) af[ks] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + ks * 32);
+#pragma unroll
+        for (int ks = 0; ks < G::kSteps; ks++) {
+          u32x4_t cur_a = af[ks % kAhead];
+          if (ks + kAhead < G::kSteps)
+            af[ks % kAhead] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + (ks + kAhead) * 32);
+          if (ks & 1) sodd = mfma32<KDT>(cur_a, qf[ks], sodd);
+          else sacc = mfma32<KDT>(cur_a, qf[ks], sacc);
+        }
+        sacc = sacc + sodd;
+      }
+      // ---- what the next unit needs, at fixed places of this unit's stream
+      if (have_next) {
+        if (t == 0) {
+          if (have_ids) request_ids(nxt, nids);
+          if (tid == 0) stop_sh[slot ^ 1] = a.n_idx;
+        }
+        if (t == 1 && have_ids) {
+          // (younger loads of this wave: the copies issued behind barrier B of the step before)
+          if (k_mine == G::kPerThread)
+            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(nids[0]), "+v"(nids[1]) : "n"(G::kPerThread) : "memory");
+          else
+            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(nids[0]), "+v"(nids[1]) : "n"(G::kPerThread - 1) : "memory");
+          scan_stop(nxt, nids, &stop_sh[slot ^ 1]);
+        }
+        if (last) request_q(nxt);  // the query registers are free from here on
+      }
+      // ---- tile s+2: of this unit, or one of the first two of the next
+      bool ahead = true;
+      int la_slot = slot, la_tile = t + 2;
+      if (la_tile >= n_cur) {
+        la_slot = slot ^ 1;
+        la_tile -= n_cur;
+        ahead = have_next;
+      }
+      uint64_t nsrc[G::kPerThread];
+      uint32_t ndst = 0;
+      if (ahead) {
+        tile_sources(la_slot, la_tile, nsrc);
+        ndst = tile_lds_base((s + 2) % G::kBufs);
+      }
+      const uint32_t mask_all = vmask[slot * 32 + t];
+      // ---- the four partial S^T of a head group meet in LDS
+      {
+        float* sxw = sx + wave * (16 * 64);
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          *reinterpret_cast<f32x4_t*>(sxw + (c * 64 + lane) * 4) =
+              f32x4_t{sacc[4 * c], sacc[4 * c + 1], sacc[4 * c + 2], sacc[4 * c + 3]};
+      }
+      lds_barrier();  // B
+      if (ahead) issue_copies(nsrc, ndst);
+      if (have_next && t == 1) {
+        const int stop_pos = stop_sh[slot ^ 1];
+        n_nxt = __builtin_amdgcn_readfirstlane(tiles_of(nxt, stop_pos));
+        build_table(nxt, slot ^ 1, nids, stop_pos, n_nxt);
+      }
+      // ---- this wave's keys 8 dh + 4 g + j: sum of the four quarters in a fixed order, softmax weights
+      float sv[4];
+      {
+        const float* sxp = sx + (hg * 4) * (16 * 64) + (dh * 64 + lane) * 4;
+        const f32x4_t p0 = *reinterpret_cast<const f32x4_t*>(sxp);
+        const f32x4_t p1 = *reinterpret_cast<const f32x4_t*>(sxp + 16 * 64);
+        const f32x4_t p2 = *reinterpret_cast<const f32x4_t*>(sxp + 2 * 16 * 64);
+        const f32x4_t p3 = *reinterpret_cast<const f32x4_t*>(sxp + 3 * 16 * 64);
+        const f32x4_t o = ((p0 + p1) + p2) + p3;
+        const uint32_t mbits = mask_all >> (8 * dh + 4 * g);
+        sv[0] = (mbits & 1u) ? o.x * a.scale_log2 : -__builtin_inff();
+        sv[1] = (mbits & 2u) ? o.y * a.scale_log2 : -__builtin_inff();
+        sv[2] = (mbits & 4u) ? o.z * a.scale_log2 : -__builtin_inff();
+        sv[3] = (mbits & 8u) ? o.w * a.scale_log2 : -__builtin_inff();
+      }
+      const float tloc = half_wave_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
+      float pw[4];
+      {
+        const float m_safe = m_run == -__builtin_inff() ? 0.0f : m_run;
+#pragma unroll
+        for (int j = 0; j < 4; j++) pw[j] = fast_exp2(sv[j] - m_safe);
+        *reinterpret_cast<u32x2_t*>(pbuf + 16 * dh + 8 * g) = u32x2_t{pack2<KDT>(pw[0], pw[1]), pack2<KDT>(pw[2], pw[3])};
+      }
+      if (__any(tloc > m_run + kGrow) && lane == 0) flag[s & 1] = s + 1;
+      // tile s+1 complete behind this barrier: this wave's copies of it are older than everything it has
+      // requested since (copies of tile s+2, ids at tile 0, the query rows at the last tile)
+      wait_vm_dyn_and_barrier((ahead ? k_mine : 0) + (have_next && have_ids && t == 0 ? 2 : 0) +
+                              (have_next && last ? G::kSteps : 0));  // C
+      if (__builtin_amdgcn_readfirstlane(flag[s & 1]) == s + 1) {
+        // ---- a key above the common maximum: the four waves agree on a new one and write P^T again
+        if (g == 0) tmaxbuf[wave * 32 + n] = tloc;
+        lds_barrier();
+        const float* tp = tmaxbuf + (hg * 4) * 32 + n;
+        const float tmax = fmaxf(fmaxf(tp[0], tp[32]), fmaxf(tp[64], tp[96]));
+        const bool grow = tmax > m_run + kGrow;
+        if (__any(grow)) {
+          const float m_new = grow ? tmax : m_run;
+          const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
+          l_run *= alpha;
+          m_run = m_new;
+#pragma unroll
+          for (int mt = 0; mt < 4; mt++) oacc[mt] = oacc[mt] * alpha;
+        }
+        const float m_safe = m_run == -__builtin_inff() ? 0.0f : m_run;
+#pragma unroll
+        for (int j = 0; j < 4; j++) pw[j] = fast_exp2(sv[j] - m_safe);
+        *reinterpret_cast<u32x2_t*>(pbuf + 16 * dh + 8 * g) = u32x2_t{pack2<KDT>(pw[0], pw[1]), pack2<KDT>(pw[2], pw[3])};
+        lds_barrier();
+      }
+      l_run += (pw[0] + pw[1]) + (pw[2] + pw[3]);
+      // ---- O^T += V^T . P^T ; P^T of the head group from LDS, key order of the accumulator layout
+      u32x4_t pf[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(pbuf + 32 * ks + 8 * g);
+        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(pbuf + 32 * ks + 16 + 8 * g);
+        pf[ks] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+      }
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++) {
+          const unsigned char* base = kt + tr_off + (16 * ks) * G::kPitch + mt * 64;
+          s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base));
+          s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base + 8 * G::kPitch));
+          u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
+          oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
+        }
+      }
+    }
+
+    // ---- end of the unit: the denominators of the four waves meet, sink, normalise, store
+    {
+      const float l_w = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
+      if (g == 0) lbuf[wave * 32 + n] = l_w;
+      lds_barrier();
+      const float* lp = lbuf + (hg * 4) * 32 + n;
+      const float l_tot = ((lp[0] + lp[32]) + lp[64]) + lp[96];
+      // the next unit's query rows have arrived before the stores go out (only the copies issued in the last
+      // step are younger), so that no wait has to count loads across stores
+      if (have_next) await_q(k_mine);
+      const int head = cur.hb * 64 + hg * 32 + n;
+      const bool q_live = head < a.n_heads;
+      const float sink = sink_l2;
+      const float m_all = fmaxf(m_run, sink);
+      const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
+      const float w = fast_exp2(m_run - m_safe);
+      const float l = l_tot * w + fast_exp2(sink - m_safe);
+      const float f = l == 0.0f ? 0.0f : w / l;
+      if (q_live) {
+        const int64_t obase = (int64_t)cur.b * a.out_batch_stride + (int64_t)cur.t * a.out_token_stride +
+                              (int64_t)head * a.out_head_stride;
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            const float r[4] = {oacc[mt][4 * c] * f, oacc[mt][4 * c + 1] * f, oacc[mt][4 * c + 2] * f,
+                                oacc[mt][4 * c + 3] * f};
+            const int dim0 = dh * 128 + 32 * mt + 8 * c + 4 * g;
+            emit_output<MSPR_F32>(a, r, obase + dim0, dim0);
+          }
+      }
+    }
+    if (!have_next) break;
+    unit += stride;
+    if (nxt.hb != cur.hb) {  // (more than 64 heads: the wait of this load drains the copies in flight once)
+      const int head = nxt.hb * 64 + hg * 32 + n;
+      sink_l2 = head < a.n_heads ? load_sink_log2(a, head) : -__builtin_inff();
+      asm volatile("" : "+v"(sink_l2));
+    }
+    cur = nxt;
+    n_cur = n_nxt;
+    slot ^= 1;
+    mask_q(cur);
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++) oacc[mt] = f32x16_t{0};
+    m_run = -__builtin_inff();
+    l_run = 0.0f;
+  }
+}
+
 template <int ODT>
 __global__ __launch_bounds__(256) void sparse_attn_merge_kernel(SparseAttnArgs a) {
   const int tid = threadIdx.x;
@@ -867,6 +1354,42 @@ int launch_split(const SparseAttnArgs& a, hipStream_t st) {
   return MSPR_OK;
 }
 
+// The persistent prefill consumer takes float16 queries and at most PrefillGeometry::kMaxTiles tiles per token;
+// everything else goes through the split kernel, one workgroup per token.
+bool prefill_consumer_fits(const SparseAttnArgs& a, int kv_dtype, int k_dim) {
+  if (!a.prefill || kv_dtype != MSPR_F16 || k_dim != 512 || a.q_dtype != MSPR_F16 || a.rope || a.out_dtype != MSPR_F32)
+    return false;
+  if (a.subst_row || a.subst_from_params || a.pool_rows_dev) return false;
+  const int tiles = (a.n_win + kTile - 1) / kTile + (a.n_idx + kTile - 1) / kTile;
+  return tiles <= PrefillGeometry::kMaxTiles;
+}
+
+int launch_prefill_consumer(const SparseAttnArgs& a, hipStream_t st) {
+  using PG = PrefillGeometry;
+  static bool attr_set = false;
+  static int n_cus = 0;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&sparse_attn_prefill_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, PG::kLdsBytes);
+    int dev = 0;
+    if (e == hipSuccess) e = hipGetDevice(&dev);
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&n_cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || n_cus < 1) {
+      mspr_set_error("sparse attention (prefill): cannot set up the kernel: %s", hipGetErrorString(e));
+      return MSPR_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  const int n_units = a.batch * a.n_hblk;
+  dim3 grid((unsigned)(n_units < n_cus ? n_units : n_cus)), block(kThreads);
+  {
+    MsprProfScope prof(MSPR_K_SPARSE_SPLIT, st);
+    sparse_attn_prefill_kernel<<<grid, block, PG::kLdsBytes, st>>>(a);
+  }
+  MSPR_CHECK_LAUNCH("sparse attention (prefill)");
+  return MSPR_OK;
+}
+
 int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* workspace, size_t workspace_bytes_given,
                          hipStream_t st) {
   const int n_keys = a.n_win + a.n_idx;
@@ -877,16 +1400,17 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
     a.out_batch_stride = (int64_t)a.n_heads * kDV;
   }
   a.n_hblk = (a.n_heads + 63) / 64;
+  auto magic = [](int n) -> uint32_t { return n <= 1 ? 0u : (uint32_t)(((uint64_t)1 << 32) / (uint32_t)n); };
+  a.inv_hblk = magic(a.n_hblk);
+  a.inv_tokens = magic(a.n_tokens);
+  if (prefill_consumer_fits(a, kv_dtype, k_dim)) return launch_prefill_consumer(a, st);
   a.n_splits = choose_splits(a.batch * a.n_hblk, n_keys);
   a.win_per_split = (a.n_win + a.n_splits - 1) / a.n_splits;
   a.idx_per_split = (a.n_idx + a.n_splits - 1) / a.n_splits;
   const int table_slots = (a.win_per_split + kTile - 1) / kTile * kTile + (a.idx_per_split + kTile - 1) / kTile * kTile;
   MSPR_REQUIRE(table_slots <= 1024, "sparse attention: too many key slots (%d)", n_keys);
   a.direct = a.n_splits == 1;
-  auto magic = [](int n) -> uint32_t { return n <= 1 ? 0u : (uint32_t)(((uint64_t)1 << 32) / (uint32_t)n); };
   a.inv_splits = magic(a.n_splits);
-  a.inv_hblk = magic(a.n_hblk);
-  a.inv_tokens = magic(a.n_tokens);
   size_t need = workspace_bytes(a.batch, a.n_heads, n_keys);
   MSPR_REQUIRE(workspace && workspace_bytes_given >= need, "sparse attention: workspace of %zu bytes needed, %zu given",
                need, workspace_bytes_given);
