@@ -728,57 +728,75 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 // Prefill consumer: many query tokens against one ring of raw rows and one pool (float16 rows of 512).
 //
 // A workgroup is persistent: it takes every gridDim.x-th (token, head block) unit and runs their 32-slot
-// tiles as one stream through the ring of three tile buffers, so that the first rows of the next token are
+// tiles as one stream through a ring of four tile buffers, so that the first rows of the next token are
 // requested while the last tiles of the current one are multiplied. What a token needs before its first
 // tile (ids -> stop position -> row pointers; its query rows) is produced inside the tile loop of the token
 // before it: ids are requested at tile 0, the row pointer table is written at tile 1 into the other of
-// two table slots, the query operand is requested behind the last S^T product. Every token runs at least
-// kMinTiles tiles (the missing ones are fully masked), which is what makes those positions exist.
+// two table slots, the query operand is requested once the last S^T product of the current token has run.
+// Every token runs at least kMinTiles tiles (the missing ones are fully masked), which is what makes those
+// positions exist.
 //
-// The tile step differs from the split kernel's. The four waves of a head group still contract a quarter
-// of the row width each, but a wave then sums only a quarter of the keys (8 of the 32: registers 4 dh ..
-// 4 dh + 3 of the four partial S^T), takes the exponentials of those alone, and writes them as P^T in the
-// element type; every wave reads the 32 x 32 P^T block of its head group back as the B operand of
-// O^T += V^T . P^T. A quarter of the exponentials and of the exchange traffic per wave, at the price of
-// a second barrier. The running maximum has to be the same in the four waves: a wave uses the common
-// m_run as it is, and raises a flag if one of its keys exceeds it by more than kGrow; on a flagged tile
-// (always the first one of a token, rarely another) the four waves exchange their maxima, rescale, and
-// write P^T again.
+// The tile step differs from the split kernel's: no wave splits a contraction, so no partial sums are
+// exchanged. For S^T = K.Q^T the 32 keys x 64 heads of a tile are eight 16 x 16 blocks, one per wave
+// (v_mfma_f32_16x16x32_f16 over the whole row width, the query block of 16 heads in 64 registers); a wave
+// takes the exponentials of its block and writes them as P^T in the element type. For O^T = V^T.P^T a wave
+// owns 32 heads x 128 output columns as in the split kernel and reads the P^T of its heads from LDS. One
+// barrier per tile (P^T written). The running maximum of a head has to be the same in every wave that
+// touches it: a wave uses the common value as it is, and raises a flag if one of its keys exceeds it by more
+// than kGrow; on a flagged tile (always the first one of a token, rarely another) the waves exchange their
+// block maxima, rescale, and write P^T again. The matrix work of a step is V^T.P^T of tile s together with
+// K.Q^T of tile s+1, in one stretch between two barriers.
 //
-// Barriers of step s: B (partial S^T written; every wave has left the V^T reads of step s-1, so the
-// copies of tile s+2 may overwrite its buffer and are issued right behind B) and C (P^T written; every
-// wave has waited for its own copies of tile s+1 before C, so tile s+1 is complete when step s+1 starts).
+// Ring: behind barrier C of step s every wave has left the V^T reads of tile s-1, so the copies of tile
+// s+3 go into its buffer; every wave waits for its own copies of tile s+1 before C, so tile s+1 is complete
+// when K.Q^T of it starts. Vector-memory waits count younger loads only, never stores.
 // ---------------------------------------------------------------------------------------------------
 struct PrefillGeometry {
   using G = Geometry<512>;
+  static constexpr int kBufs = 4;                         // one tile under V^T.P^T, one under K.Q^T, two in flight
+  static constexpr int kSlots = 66;                       // 16-byte slots per LDS row, two of them padding: rows 32
+                                                          // bytes apart in the banks serve the 16-row operand
+                                                          // reads of K.Q^T and the transpose reads best
+  static constexpr int kPitch = kSlots * 16;
+  static constexpr int kTileSlots = kTile * kSlots;       // = 33 wave-wide copies exactly
   static constexpr int kMaxTiles = 22;                    // 704 slots per token
-  static constexpr int kMinTiles = 4;
+  static constexpr int kMinTiles = 5;
   static constexpr int kTableSlots = kMaxTiles * kTile;
+  static constexpr int kQSteps = 512 / 32;                // MFMAs of one 16 x 16 block of S^T
   static constexpr int kPPitch = 80;                      // bytes per head of P^T: 32 keys + 16 B, so that the
-                                                          // 16 heads of a read phase start on distinct banks
-  static constexpr int kOffSx = G::kBufs * G::kTileBytes;            // [8 waves][4 key octets][64 lanes][4] float
-  static constexpr int kOffTable = kOffSx + kWaves * 4096;           // [2][kTableSlots] row pointers
+                                                          // heads of a read phase start on distinct banks
+  static constexpr int kOffTable = kBufs * G::kTileBytes;            // [2][kTableSlots] row pointers
   static constexpr int kOffVmask = kOffTable + 2 * kTableSlots * 8;  // [2][32] validity word per tile
-  static constexpr int kOffP = kOffVmask + 2 * 32 * 4;               // [2 head groups][32 heads][kPPitch]
-  static constexpr int kOffTmax = kOffP + 2 * 32 * kPPitch;          // [8 waves][32 heads] float
-  static constexpr int kOffL = kOffTmax + kWaves * 32 * 4;           // [8 waves][32 heads] float
-  static constexpr int kOffFlag = kOffL + kWaves * 32 * 4;           // flag[2], stop[2]
-  static constexpr int kLdsBytes = kOffFlag + 16;
-  static_assert(kOffTable % 16 == 0 && kOffP % 16 == 0 && kLdsBytes <= 160 * 1024, "LDS map of the prefill consumer");
+  static constexpr int kOffP = kOffVmask + 2 * 32 * 4;               // [2 steps][64 heads][kPPitch]
+  static constexpr int kOffTmax = kOffP + 2 * 64 * kPPitch;          // [8 waves][16 heads] float
+  static constexpr int kOffL = kOffTmax + kWaves * 16 * 4;           // [8 waves][16 heads] float
+  static constexpr int kOffFlag = kOffL + kWaves * 16 * 4;           // flag[2], stop[2]
+  static constexpr int kOffWarm = kOffFlag + 16;                     // [8 waves][64 lanes] dwords nobody reads
+  static constexpr int kLdsBytes = kOffWarm + kWaves * 256;
+  static_assert(kTileSlots == G::kInstr * 64 && kOffTable % 16 == 0 && kOffP % 16 == 0 && kLdsBytes <= 160 * 1024, "LDS map of the prefill consumer");
 };
 
-// s_waitcnt vmcnt(n) for a wave-uniform n (the encodable counts that the prefill kernel needs), then the
-// LDS wait and the barrier
+__device__ __forceinline__ f32x4_t mfma16_f16(u32x4_t a, u32x4_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0,
+                                                0);
+}
+
+// s_waitcnt vmcnt(n) for a wave-uniform n (the counts that the prefill kernel can ask for; anything else waits
+// for everything), then the LDS wait and the barrier
 __device__ __forceinline__ void wait_vm_dyn_and_barrier(int n) {
   switch (n) {
-    case 2: wait_vm_and_barrier<2>(); break;
     case 4: wait_vm_and_barrier<4>(); break;
     case 5: wait_vm_and_barrier<5>(); break;
     case 6: wait_vm_and_barrier<6>(); break;
     case 7: wait_vm_and_barrier<7>(); break;
     case 8: wait_vm_and_barrier<8>(); break;
-    case 12: wait_vm_and_barrier<12>(); break;
-    case 13: wait_vm_and_barrier<13>(); break;
+    case 10: wait_vm_and_barrier<10>(); break;
+    case 20: wait_vm_and_barrier<20>(); break;
+    case 21: wait_vm_and_barrier<21>(); break;
+    case 22: wait_vm_and_barrier<22>(); break;
+    case 23: wait_vm_and_barrier<23>(); break;
+    case 38: wait_vm_and_barrier<38>(); break;
+    case 39: wait_vm_and_barrier<39>(); break;
     default: wait_vm_and_barrier<0>(); break;
   }
 }
@@ -796,7 +814,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
   using PG = PrefillGeometry;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   unsigned char* kbuf = lds;
-  float* sx = reinterpret_cast<float*>(lds + PG::kOffSx);
   uint64_t* table = reinterpret_cast<uint64_t*>(lds + PG::kOffTable);
   uint32_t* vmask = reinterpret_cast<uint32_t*>(lds + PG::kOffVmask);
   float* tmaxbuf = reinterpret_cast<float*>(lds + PG::kOffTmax);
@@ -807,11 +824,19 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  // O^T = V^T.P^T: wave = (head group of 32, quarter of the output columns), lane = (head n, half g)
   const int hg = wave >> 2;
   const int dh = wave & 3;
   const int n = lane & 31;
   const int g = lane >> 5;
-  unsigned char* pbuf = lds + PG::kOffP + hg * (32 * PG::kPPitch) + n * PG::kPPitch;
+  // S^T = K.Q^T: wave = (key half, head quarter), lane = (row / column c16 of the block, k group kg)
+  const int kh = wave & 1;
+  const int hq = wave >> 1;
+  const int c16 = lane & 15;
+  const int kg = lane >> 4;
+  unsigned char* p_wr = lds + PG::kOffP + (16 * hq + c16) * PG::kPPitch + 32 * kh + 8 * kg;  // keys 16 kh + 4 kg ..
+  const unsigned char* p_rd = lds + PG::kOffP + (32 * hg + n) * PG::kPPitch + 8 * g;
+  const int tmax_rd = (2 * (2 * hg + (n >> 4))) * 16 + (n & 15);  // first of the two blocks that hold head 32 hg + n
   const int k_mine = wave < G::kLastWaves ? G::kPerThread : G::kPerThread - 1;  // copies of this wave per tile
 
   const int n_units = a.batch * a.n_hblk;
@@ -913,61 +938,69 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
 #pragma unroll
   for (int j = 0; j < G::kPerThread; j++) {
     const int P = tid + kThreads * j;
-    const int row = P / G::kSlots, chunk = P % G::kSlots;
-    pk[j] = (P < G::kTileSlots && chunk != G::kSlots - 1) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
+    const int row = P / PG::kSlots, chunk = P % PG::kSlots;
+    pk[j] = (P < PG::kTileSlots && chunk < 64) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
   }
-  auto tile_sources = [&](int slot, int tile, uint64_t (&src)[G::kPerThread]) {
+  auto copy_tile = [&](int slot, int tile, int buf) {
     const uint64_t* rp = table + slot * PG::kTableSlots + tile * kTile;
+    uint64_t src[G::kPerThread];
 #pragma unroll
     for (int j = 0; j < G::kPerThread; j++) {
       const uint32_t p = pk[j];
       const bool act = p != 0xFFFFFFFFu;
       src[j] = rp[act ? (p >> 16) : 0] + (act ? (p & 0xFFFFu) : 0u);
     }
-  };
-  auto tile_lds_base = [&](int buf) -> uint32_t {
-    return __builtin_amdgcn_readfirstlane(
+    const uint32_t dst_lds = __builtin_amdgcn_readfirstlane(
         (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, kbuf + buf * G::kTileBytes + wave * 1024));
-  };
-  auto issue_copies = [&](const uint64_t (&src)[G::kPerThread], uint32_t dst_lds) {
 #pragma unroll
     for (int j = 0; j < G::kPerThread; j++)
       if (j < G::kPerThread - 1 || wave < G::kLastWaves) async_load_16(src[j], dst_lds + j * (kWaves * 1024));
   };
 
-  // ---- query operand of a unit: lane (n = head, g) holds q[head][dh*128 + 16 ks + 8 g .. +7]
-  u32x4_t qf[G::kSteps];
+  // ---- query operand of a unit: lane (c16 = head of the quarter, kg) holds q[head][32 ks + 8 kg .. +7]
+  u32x4_t qf[PG::kQSteps];
   auto request_q = [&](const PrefillUnit& m) {
-    const int head = m.hb * 64 + hg * 32 + n;
+    const int head = m.hb * 64 + 16 * hq + c16;
     const int64_t qoff = (int64_t)m.b * a.q_batch_stride + (int64_t)m.t * a.q_token_stride +
-                         (int64_t)(head < a.n_heads ? head : 0) * a.q_head_stride + dh * G::kPart + 8 * g;
+                         (int64_t)(head < a.n_heads ? head : 0) * a.q_head_stride + 8 * kg;
     const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
 #pragma unroll
-    for (int ks = 0; ks < G::kSteps; ks++) {
-      const uint16_t* p = qp + 16 * ks;
+    for (int ks = 0; ks < PG::kQSteps; ks++) {
+      const uint16_t* p = qp + 32 * ks;
       asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(qf[ks]) : "v"(p) : "memory");
     }
   };
-  static_assert(G::kSteps == 8, "the query wait below names eight registers");
-  auto await_q = [&](int newer) {  // at most `newer` younger loads of this wave may stay in flight
-    if (newer == G::kPerThread)
-      asm volatile("s_waitcnt vmcnt(%8)" : "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]),
-                   "+v"(qf[6]), "+v"(qf[7]) : "n"(G::kPerThread) : "memory");
-    else if (newer == G::kPerThread - 1)
-      asm volatile("s_waitcnt vmcnt(%8)" : "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]),
-                   "+v"(qf[6]), "+v"(qf[7]) : "n"(G::kPerThread - 1) : "memory");
-    else
-      asm volatile("s_waitcnt vmcnt(0)" : "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]),
-                   "+v"(qf[6]), "+v"(qf[7]) : : "memory");
+  // one dword of every 128-byte line of a unit's query rows (64 rows of 1 KB), requested long before the rows
+  // themselves so that those come out of the L2. The dwords go to LDS nobody reads: a load into a register
+  // that is dead behind the request would land in whatever the register holds by then.
+  const uint32_t warm_lds = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, lds + PG::kOffWarm + wave * 256));
+  auto warm_q = [&](const PrefillUnit& m) {
+    const int head = m.hb * 64 + (tid >> 3);
+    const uint16_t* p = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)m.b * a.q_batch_stride +
+                        (int64_t)m.t * a.q_token_stride + (int64_t)(head < a.n_heads ? head : 0) * a.q_head_stride +
+                        (tid & 7) * 64;
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(p), "s"(warm_lds) : "memory", "m0");
   };
+  static_assert(PG::kQSteps == 16, "the query wait below names sixteen registers");
+#define MSPR_QF_OPERANDS                                                                                             \
+  "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]), "+v"(qf[6]), "+v"(qf[7]), "+v"(qf[8]), \
+      "+v"(qf[9]), "+v"(qf[10]), "+v"(qf[11]), "+v"(qf[12]), "+v"(qf[13]), "+v"(qf[14]), "+v"(qf[15])
+  auto await_q = [&](int newer) {  // at most `newer` younger loads of this wave may stay in flight
+    if (newer == G::kPerThread) asm volatile("s_waitcnt vmcnt(%16)" : MSPR_QF_OPERANDS : "n"(G::kPerThread) : "memory");
+    else if (newer == G::kPerThread - 1)
+      asm volatile("s_waitcnt vmcnt(%16)" : MSPR_QF_OPERANDS : "n"(G::kPerThread - 1) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" : MSPR_QF_OPERANDS : : "memory");
+  };
+#undef MSPR_QF_OPERANDS
   auto mask_q = [&](const PrefillUnit& m) {
-    if (m.hb * 64 + hg * 32 + n >= a.n_heads) {
+    if (m.hb * 64 + 16 * hq + c16 >= a.n_heads) {
 #pragma unroll
-      for (int ks = 0; ks < G::kSteps; ks++) qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
+      for (int ks = 0; ks < PG::kQSteps; ks++) qf[ks] = u32x4_t{0u, 0u, 0u, 0u};
     }
   };
 
-  // ---- first unit: ids, stop position, table, query, first two tiles
+  // ---- first unit: ids, stop position, table, query, first three tiles
   PrefillUnit cur = unit_of(unit);
   int ids[2];
   const bool have_ids = a.n_idx > 0;
@@ -976,7 +1009,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
   if (tid == 0) stop_sh[0] = a.n_idx;
   __syncthreads();
   if (have_ids) {
-    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(ids[0]), "+v"(ids[1]) : "n"(G::kSteps) : "memory");
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(ids[0]), "+v"(ids[1]) : "n"(PG::kQSteps) : "memory");
     scan_stop(cur, ids, &stop_sh[0]);
   }
   __syncthreads();
@@ -992,30 +1025,49 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     asm volatile("" : "+v"(sink_l2));
   }
   __syncthreads();
-  {
-    uint64_t src[G::kPerThread];
-    tile_sources(0, 0, src);
-    issue_copies(src, tile_lds_base(0));
-    tile_sources(0, 1, src);
-    issue_copies(src, tile_lds_base(1));
-  }
+  copy_tile(0, 0, 0);
+  copy_tile(0, 1, 1);
+  copy_tile(0, 2, 2);
 
   f32x16_t oacc[4];
 #pragma unroll
   for (int mt = 0; mt < 4; mt++) oacc[mt] = f32x16_t{0};
-  float m_run = -__builtin_inff();  // reference maximum per head, the same in the four waves of a head group
-  float l_run = 0.0f;               // this wave's keys only
+  // reference maximum per head, the same in every wave that holds the head: m_qk for head 16 hq + c16 (S^T
+  // role), m_pv for head 32 hg + n (O^T role)
+  float m_qk = -__builtin_inff(), m_pv = -__builtin_inff();
+  float l_qk = 0.0f;  // denominator share of this lane: its head, its four keys of every tile
 
-  const int a_row_off = n * G::kPitch + (dh * G::kPart + 8 * g) * 2;
+  const int a_row_off = (16 * kh + c16) * PG::kPitch + 16 * kg;
   const int tr_s = lane & 15;
-  const int tr_off = (4 * g + (tr_s >> 2)) * G::kPitch + (dh * 128 + 16 * ((lane >> 4) & 1) + 4 * (tr_s & 3)) * 2;
+  const int tr_off = (4 * g + (tr_s >> 2)) * PG::kPitch + (dh * 128 + 16 * ((lane >> 4) & 1) + 4 * (tr_s & 3)) * 2;
   constexpr float kGrow = 8.0f;  // float16 weights stay below 2^15
 
-  // tile 0 is complete once every wave's copies of it are (the copies of tile 1 stay in flight)
-  wait_vm_dyn_and_barrier(k_mine);
+  // S^T block of one tile
+  auto qk_block = [&](const unsigned char* kt) -> f32x4_t {
+    f32x4_t se = {0.0f, 0.0f, 0.0f, 0.0f}, so = {0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int kAhead = 6;
+    u32x4_t af[kAhead];
+#pragma unroll
+    for (int ks = 0; ks < kAhead; ks++) af[ks] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + ks * 64);
+#pragma unroll
+    for (int ks = 0; ks < PG::kQSteps; ks++) {
+      const u32x4_t cur_a = af[ks % kAhead];
+      if (ks + kAhead < PG::kQSteps)
+        af[ks % kAhead] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + (ks + kAhead) * 64);
+      if (ks & 1) so = mfma16_f16(cur_a, qf[ks], so);
+      else se = mfma16_f16(cur_a, qf[ks], se);
+    }
+    return se + so;
+  };
 
-  int s = 0;    // tiles done by this workgroup: ring buffer s % 3, flag slot s & 1
-  int slot = 0; // table slot of the current unit
+  // tile 0 is complete once every wave's copies of it are (the copies of tiles 1 and 2 stay in flight)
+  wait_vm_dyn_and_barrier(2 * k_mine);
+  f32x4_t sacc = qk_block(kbuf);
+
+  int s = 0;           // tiles done by this workgroup: ring buffer s % 4, flag and P^T slot s & 1
+  int slot = 0;        // table slot of the current unit
+  int prev_extra = 0;  // loads other than tile copies that this wave requested in the step before
+  int stores_behind = 0;  // output stores of the unit before (16 per wave that holds a live head)
   for (;;) {
     const bool have_next = unit + stride < n_units;
     PrefillUnit nxt = cur;
@@ -1024,159 +1076,146 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     if (have_next) nxt = unit_of(unit + stride);
 
     for (int t = 0; t < n_cur; t++, s++) {
-      const unsigned char* kt = kbuf + (s % G::kBufs) * G::kTileBytes;
       const bool last = t == n_cur - 1;
-      // ---- S^T partial over this wave's quarter of the row width (two chains of dependent MFMAs)
-      f32x16_t sacc = {0};
-      {
-        f32x16_t sodd = {0};
-        constexpr int kAhead = 6;
-        u32x4_t af[kAhead];
-#pragma unroll
-        for (int ks = 0; ks < kAhead; ks++) af[ks] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + ks * 32);
-#pragma unroll
-        for (int ks = 0; ks < G::kSteps; ks++) {
-          u32x4_t cur_a = af[ks % kAhead];
-          if (ks + kAhead < G::kSteps)
-            af[ks % kAhead] = *reinterpret_cast<const u32x4_t*>(kt + a_row_off + (ks + kAhead) * 32);
-          if (ks & 1) sodd = mfma32<KDT>(cur_a, qf[ks], sodd);
-          else sacc = mfma32<KDT>(cur_a, qf[ks], sacc);
-        }
-        sacc = sacc + sodd;
-      }
       // ---- what the next unit needs, at fixed places of this unit's stream
+      int extra = 0;
       if (have_next) {
-        if (t == 0) {
-          if (have_ids) request_ids(nxt, nids);
-          if (tid == 0) stop_sh[slot ^ 1] = a.n_idx;
-        }
         if (t == 1 && have_ids) {
-          // (younger loads of this wave: the copies issued behind barrier B of the step before)
+          // (younger loads of this wave: the copies issued behind barrier C of the step before)
           if (k_mine == G::kPerThread)
             asm volatile("s_waitcnt vmcnt(%2)" : "+v"(nids[0]), "+v"(nids[1]) : "n"(G::kPerThread) : "memory");
           else
             asm volatile("s_waitcnt vmcnt(%2)" : "+v"(nids[0]), "+v"(nids[1]) : "n"(G::kPerThread - 1) : "memory");
           scan_stop(nxt, nids, &stop_sh[slot ^ 1]);
         }
-        if (last) request_q(nxt);  // the query registers are free from here on
+        if (t == 0) {
+          if (have_ids) {
+            request_ids(nxt, nids);
+            extra = 2;
+          }
+          if (tid == 0) stop_sh[slot ^ 1] = a.n_idx;
+        }
+        if (t == 2) {
+          warm_q(nxt);
+          extra = 1;
+        }
+        if (last) {  // K.Q^T of this unit's last tile ran in the step before: the query registers are free
+          request_q(nxt);
+          extra = PG::kQSteps;
+        }
       }
-      // ---- tile s+2: of this unit, or one of the first two of the next
-      bool ahead = true;
-      int la_slot = slot, la_tile = t + 2;
-      if (la_tile >= n_cur) {
-        la_slot = slot ^ 1;
-        la_tile -= n_cur;
-        ahead = have_next;
-      }
-      uint64_t nsrc[G::kPerThread];
-      uint32_t ndst = 0;
-      if (ahead) {
-        tile_sources(la_slot, la_tile, nsrc);
-        ndst = tile_lds_base((s + 2) % G::kBufs);
-      }
-      const uint32_t mask_all = vmask[slot * 32 + t];
-      // ---- the four partial S^T of a head group meet in LDS
+      // ---- softmax weights of this wave's block: head 16 hq + c16, keys 16 kh + 4 kg + i
+      float sv[4];
       {
-        float* sxw = sx + wave * (16 * 64);
-#pragma unroll
-        for (int c = 0; c < 4; c++)
-          *reinterpret_cast<f32x4_t*>(sxw + (c * 64 + lane) * 4) =
-              f32x4_t{sacc[4 * c], sacc[4 * c + 1], sacc[4 * c + 2], sacc[4 * c + 3]};
+        const uint32_t mbits = vmask[slot * 32 + t] >> (16 * kh + 4 * kg);
+        sv[0] = (mbits & 1u) ? sacc[0] * a.scale_log2 : -__builtin_inff();
+        sv[1] = (mbits & 2u) ? sacc[1] * a.scale_log2 : -__builtin_inff();
+        sv[2] = (mbits & 4u) ? sacc[2] * a.scale_log2 : -__builtin_inff();
+        sv[3] = (mbits & 8u) ? sacc[3] * a.scale_log2 : -__builtin_inff();
       }
-      lds_barrier();  // B
-      if (ahead) issue_copies(nsrc, ndst);
+      const float tloc = half_wave_max(row_pair_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]))));
+      float pw[4];
+      unsigned char* p_wr_s = p_wr + (s & 1) * (64 * PG::kPPitch);
+      {
+        const float m_safe = m_qk == -__builtin_inff() ? 0.0f : m_qk;
+#pragma unroll
+        for (int j = 0; j < 4; j++) pw[j] = fast_exp2(sv[j] - m_safe);
+        *reinterpret_cast<u32x2_t*>(p_wr_s) = u32x2_t{pack2<KDT>(pw[0], pw[1]), pack2<KDT>(pw[2], pw[3])};
+      }
+      if (__any(tloc > m_qk + kGrow) && lane == 0) flag[s & 1] = s + 1;
+      // tile s+1 complete behind this barrier: this wave's copies of it are older than everything it has
+      // requested since (the copies of tile s+2, and ids or query rows in this step and the one before)
+      const bool two_ahead = t + 2 < n_cur || have_next;
+      // (the stores of the unit before are younger than the awaited copies in its first two steps; loads and
+      // stores of a wave complete in the order issued)
+      wait_vm_dyn_and_barrier(prev_extra + (two_ahead ? k_mine : 0) + extra + (t < 2 ? stores_behind : 0));  // C
+      prev_extra = extra;
+      if (__builtin_amdgcn_readfirstlane(flag[s & 1]) == s + 1) {
+        // ---- a key above the common maximum: the waves agree on a new one and write P^T again
+        if (kg == 0) tmaxbuf[wave * 16 + c16] = tloc;
+        lds_barrier();
+        {
+          const float tq = fmaxf(tmaxbuf[(2 * hq) * 16 + c16], tmaxbuf[(2 * hq + 1) * 16 + c16]);
+          const bool grow = tq > m_qk + kGrow;
+          l_qk *= grow ? fast_exp2(m_qk - tq) : 1.0f;
+          m_qk = grow ? tq : m_qk;
+        }
+        {
+          const float tp = fmaxf(tmaxbuf[tmax_rd], tmaxbuf[tmax_rd + 16]);
+          const bool grow = tp > m_pv + kGrow;
+          if (__any(grow)) {
+            const float alpha = grow ? fast_exp2(m_pv - tp) : 1.0f;
+            m_pv = grow ? tp : m_pv;
+#pragma unroll
+            for (int mt = 0; mt < 4; mt++) oacc[mt] = oacc[mt] * alpha;
+          }
+        }
+        const float m_safe = m_qk == -__builtin_inff() ? 0.0f : m_qk;
+#pragma unroll
+        for (int j = 0; j < 4; j++) pw[j] = fast_exp2(sv[j] - m_safe);
+        *reinterpret_cast<u32x2_t*>(p_wr_s) = u32x2_t{pack2<KDT>(pw[0], pw[1]), pack2<KDT>(pw[2], pw[3])};
+        lds_barrier();
+      }
+      l_qk += (pw[0] + pw[1]) + (pw[2] + pw[3]);
+      // ---- tile s+3: of this unit, or one of the first three of the next
+      {
+        int la_slot = slot, la_tile = t + 3;
+        bool ahead = true;
+        if (la_tile >= n_cur) {
+          la_slot = slot ^ 1;
+          la_tile -= n_cur;
+          ahead = have_next;
+        }
+        if (ahead) copy_tile(la_slot, la_tile, (s + 3) % PG::kBufs);
+      }
       if (have_next && t == 1) {
         const int stop_pos = stop_sh[slot ^ 1];
         n_nxt = __builtin_amdgcn_readfirstlane(tiles_of(nxt, stop_pos));
         build_table(nxt, slot ^ 1, nids, stop_pos, n_nxt);
       }
-      // ---- this wave's keys 8 dh + 4 g + j: sum of the four quarters in a fixed order, softmax weights
-      float sv[4];
-      {
-        const float* sxp = sx + (hg * 4) * (16 * 64) + (dh * 64 + lane) * 4;
-        const f32x4_t p0 = *reinterpret_cast<const f32x4_t*>(sxp);
-        const f32x4_t p1 = *reinterpret_cast<const f32x4_t*>(sxp + 16 * 64);
-        const f32x4_t p2 = *reinterpret_cast<const f32x4_t*>(sxp + 2 * 16 * 64);
-        const f32x4_t p3 = *reinterpret_cast<const f32x4_t*>(sxp + 3 * 16 * 64);
-        const f32x4_t o = ((p0 + p1) + p2) + p3;
-        const uint32_t mbits = mask_all >> (8 * dh + 4 * g);
-        sv[0] = (mbits & 1u) ? o.x * a.scale_log2 : -__builtin_inff();
-        sv[1] = (mbits & 2u) ? o.y * a.scale_log2 : -__builtin_inff();
-        sv[2] = (mbits & 4u) ? o.z * a.scale_log2 : -__builtin_inff();
-        sv[3] = (mbits & 8u) ? o.w * a.scale_log2 : -__builtin_inff();
+      if (have_next && last) {
+        await_q(k_mine);  // (younger: the copies issued just above)
+        mask_q(nxt);
       }
-      const float tloc = half_wave_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
-      float pw[4];
-      {
-        const float m_safe = m_run == -__builtin_inff() ? 0.0f : m_run;
-#pragma unroll
-        for (int j = 0; j < 4; j++) pw[j] = fast_exp2(sv[j] - m_safe);
-        *reinterpret_cast<u32x2_t*>(pbuf + 16 * dh + 8 * g) = u32x2_t{pack2<KDT>(pw[0], pw[1]), pack2<KDT>(pw[2], pw[3])};
-      }
-      if (__any(tloc > m_run + kGrow) && lane == 0) flag[s & 1] = s + 1;
-      // tile s+1 complete behind this barrier: this wave's copies of it are older than everything it has
-      // requested since (copies of tile s+2, ids at tile 0, the query rows at the last tile)
-      wait_vm_dyn_and_barrier((ahead ? k_mine : 0) + (have_next && have_ids && t == 0 ? 2 : 0) +
-                              (have_next && last ? G::kSteps : 0));  // C
-      if (__builtin_amdgcn_readfirstlane(flag[s & 1]) == s + 1) {
-        // ---- a key above the common maximum: the four waves agree on a new one and write P^T again
-        if (g == 0) tmaxbuf[wave * 32 + n] = tloc;
-        lds_barrier();
-        const float* tp = tmaxbuf + (hg * 4) * 32 + n;
-        const float tmax = fmaxf(fmaxf(tp[0], tp[32]), fmaxf(tp[64], tp[96]));
-        const bool grow = tmax > m_run + kGrow;
-        if (__any(grow)) {
-          const float m_new = grow ? tmax : m_run;
-          const float alpha = grow ? fast_exp2(m_run - m_new) : 1.0f;
-          l_run *= alpha;
-          m_run = m_new;
-#pragma unroll
-          for (int mt = 0; mt < 4; mt++) oacc[mt] = oacc[mt] * alpha;
-        }
-        const float m_safe = m_run == -__builtin_inff() ? 0.0f : m_run;
-#pragma unroll
-        for (int j = 0; j < 4; j++) pw[j] = fast_exp2(sv[j] - m_safe);
-        *reinterpret_cast<u32x2_t*>(pbuf + 16 * dh + 8 * g) = u32x2_t{pack2<KDT>(pw[0], pw[1]), pack2<KDT>(pw[2], pw[3])};
-        lds_barrier();
-      }
-      l_run += (pw[0] + pw[1]) + (pw[2] + pw[3]);
-      // ---- O^T += V^T . P^T ; P^T of the head group from LDS, key order of the accumulator layout
+      // ---- O^T += V^T . P^T of tile s, and S^T of tile s+1
+      const unsigned char* kt = kbuf + (s % PG::kBufs) * G::kTileBytes;
+      const unsigned char* p_rd_s = p_rd + (s & 1) * (64 * PG::kPPitch);
       u32x4_t pf[2];
 #pragma unroll
       for (int ks = 0; ks < 2; ks++) {
-        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(pbuf + 32 * ks + 8 * g);
-        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(pbuf + 32 * ks + 16 + 8 * g);
+        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(p_rd_s + 32 * ks);
+        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(p_rd_s + 32 * ks + 16);
         pf[ks] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
       }
 #pragma unroll
       for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
         for (int mt = 0; mt < 4; mt++) {
-          const unsigned char* base = kt + tr_off + (16 * ks) * G::kPitch + mt * 64;
+          const unsigned char* base = kt + tr_off + (16 * ks) * PG::kPitch + mt * 64;
           s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base));
-          s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base + 8 * G::kPitch));
+          s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base + 8 * PG::kPitch));
           u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
           oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
         }
       }
+      if (!last || have_next) sacc = qk_block(kbuf + ((s + 1) % PG::kBufs) * G::kTileBytes);
     }
 
-    // ---- end of the unit: the denominators of the four waves meet, sink, normalise, store
+    // ---- end of the unit: the denominators meet, sink, normalise, store
     {
-      const float l_w = l_run + __shfl_xor(l_run, 32, MSPR_WAVE);
-      if (g == 0) lbuf[wave * 32 + n] = l_w;
+      float l_w = l_qk;
+      l_w += __shfl_xor(l_w, 16, MSPR_WAVE);
+      l_w += __shfl_xor(l_w, 32, MSPR_WAVE);
+      if (kg == 0) lbuf[wave * 16 + c16] = l_w;
       lds_barrier();
-      const float* lp = lbuf + (hg * 4) * 32 + n;
-      const float l_tot = ((lp[0] + lp[32]) + lp[64]) + lp[96];
-      // the next unit's query rows have arrived before the stores go out (only the copies issued in the last
-      // step are younger), so that no wait has to count loads across stores
-      if (have_next) await_q(k_mine);
+      const float l_tot = lbuf[tmax_rd] + lbuf[tmax_rd + 16];
       const int head = cur.hb * 64 + hg * 32 + n;
       const bool q_live = head < a.n_heads;
+      stores_behind = __any(q_live) ? 16 : 0;
       const float sink = sink_l2;
-      const float m_all = fmaxf(m_run, sink);
+      const float m_all = fmaxf(m_pv, sink);
       const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
-      const float w = fast_exp2(m_run - m_safe);
+      const float w = fast_exp2(m_pv - m_safe);
       const float l = l_tot * w + fast_exp2(sink - m_safe);
       const float f = l == 0.0f ? 0.0f : w / l;
       if (q_live) {
@@ -1203,11 +1242,11 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     cur = nxt;
     n_cur = n_nxt;
     slot ^= 1;
-    mask_q(cur);
 #pragma unroll
     for (int mt = 0; mt < 4; mt++) oacc[mt] = f32x16_t{0};
-    m_run = -__builtin_inff();
-    l_run = 0.0f;
+    m_qk = -__builtin_inff();
+    m_pv = -__builtin_inff();
+    l_qk = 0.0f;
   }
 }
 
