@@ -336,6 +336,14 @@ def bench_ds4_prefill(dev, gen, reps=5):
     return out
 
 
+def guarded(leg, *args, **kwargs):
+    """A side leg of the benchmark: its failure is reported in its place and leaves the headline line intact."""
+    try:
+        return leg(*args, **kwargs)
+    except Exception as exc:  # noqa: BLE001 - whatever a leg raises belongs in the report, not in the exit code
+        return {"error": f"{type(exc).__name__}: {exc}"[:300]}
+
+
 def calibration_copy(dev):
     """One elementwise kernel that reads 1 GiB and writes 1 GiB: the scale of the HBM byte counters."""
     src = torch.ones(1 << 28, device=dev, dtype=torch.float32)
@@ -498,13 +506,13 @@ def main() -> int:
     extras = {
         "kernel_us": {k: round(v, 2) for k, v in kernel_us.items()},
         "kernel_us_by_batch": by_batch,
-        "prefill": None if args.headline_only else bench_prefill(dev, gen),
-        "prefill_q8": None if args.headline_only else bench_prefill_q8(dev, gen),
-        "q8_decode": None if args.headline_only else bench_q8_decode(dev, gen),
-        "ds4_prefill": None if args.headline_only else bench_ds4_prefill(dev, gen),
-        "cpu_config1": None if args.no_cpu_baseline else cpu_config1(),
-        "cpu_configs_2_3": None if args.no_cpu_baseline else cpu_other_configs(),
-        "cpu_baseline_1thread": None if args.no_cpu_baseline else cpu_baseline(seconds_budget=6.0, threads=1),
+        "prefill": None if args.headline_only else guarded(bench_prefill, dev, gen),
+        "prefill_q8": None if args.headline_only else guarded(bench_prefill_q8, dev, gen),
+        "q8_decode": None if args.headline_only else guarded(bench_q8_decode, dev, gen),
+        "ds4_prefill": None if args.headline_only else guarded(bench_ds4_prefill, dev, gen),
+        "cpu_config1": None if args.no_cpu_baseline else guarded(cpu_config1),
+        "cpu_configs_2_3": None if args.no_cpu_baseline else guarded(cpu_other_configs),
+        "cpu_baseline_1thread": None if args.no_cpu_baseline else guarded(cpu_baseline, seconds_budget=6.0, threads=1),
         "indexer_fp8_GBps": round(IDX_BYTES_PER_SEQ * B / (kernel_us["indexer_fp8"] * 1e-6) / 1e9, 1),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
         "buffer_sets": R,
