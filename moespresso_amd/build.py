@@ -66,5 +66,38 @@ def build(verbose: bool = True) -> str:
     return LIB_PATH
 
 
+def kernel_resources(src: str) -> dict[str, dict[str, int]]:
+    """Registers and scratch of every kernel in one HIP source, from the code object metadata of a device-only
+    compile to assembly: ``{kernel symbol: {"vgprs", "sgprs", "scratch_bytes", "vgpr_spills", "sgpr_spills"}}``.
+
+    The kernels that count their own vector-memory operations (asynchronous tile copies awaited with
+    ``s_waitcnt vmcnt(n)``) rely on the compiler adding none: a register spilled to scratch is one more
+    vector-memory operation in the middle of the count, and its reload drains every copy in flight.
+    """
+    import re
+    import tempfile
+
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "kernels.s")
+        cmd = [HIPCC, *COMMON_FLAGS, "-S", "--cuda-device-only", "-o", out, src]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{proc.stderr}")
+        text = open(out).read()
+    fields = {"vgprs": "vgpr_count", "sgprs": "sgpr_count", "scratch_bytes": "private_segment_fixed_size",
+              "vgpr_spills": "vgpr_spill_count", "sgpr_spills": "sgpr_spill_count"}
+    kernels: dict[str, dict[str, int]] = {}
+    # one metadata record per kernel: "- .agpr_count: ..." up to the next record; ".name:" carries the symbol
+    for record in re.split(r"\n  - \.", text[text.index("amdhsa.kernels:"):])[1:]:
+        name = re.search(r"\.name:\s+(\S+)", record)
+        if not name:
+            continue
+        kernels[name.group(1)] = {
+            key: int(m.group(1)) if (m := re.search(rf"\.{field}:\s+(\d+)", record)) else 0
+            for key, field in fields.items()
+        }
+    return kernels
+
+
 if __name__ == "__main__":
     build()
