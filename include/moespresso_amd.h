@@ -159,7 +159,8 @@ int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, const void*
  * (top_k may be 0); sinks: f32 [n_heads]; out: f32 with the strides of q.
  * Float16 queries whose slot count fits 22 tiles of 32 (window and ids each rounded up to whole tiles) run on
  * one persistent workgroup per CU that streams consecutive tokens; other calls take one workgroup per token and
- * key range. The arguments and the workspace size asked for are the same either way.
+ * key range (every call does with MSPR_PREFILL_PERSISTENT=0 in the environment, read per call). The arguments
+ * and the workspace size asked for are the same either way.
  * Workspace: mspr_sparse_attention_workspace_bytes(batch*n_tokens, n_heads, min(window or raw_cap, raw_cap) + top_k). */
 int mspr_indexed_mixed_attention_prefill(const void* q, int q_dtype, int batch, int n_heads, int n_tokens,
                                          int64_t q_batch_stride, int64_t q_head_stride,

@@ -25,6 +25,8 @@
 #include "common.h"
 #include "profile.h"
 
+#include <cstdlib>
+
 // Scratch of mspr_sparse_mla_decode_static, the entry point that allocates nothing: the partials of up to 256
 // key ranges (a grid of one workgroup per CU), 64 heads x 512 float16 and 64 x (m, l) float32 each. Every range
 // of a call is written before it is read, so nothing in it has to start at zero. Host code never uses this
@@ -1398,6 +1400,10 @@ int launch_split(const SparseAttnArgs& a, hipStream_t st) {
 bool prefill_consumer_fits(const SparseAttnArgs& a, int kv_dtype, int k_dim) {
   if (!a.prefill || kv_dtype != MSPR_F16 || k_dim != 512 || a.q_dtype != MSPR_F16 || a.rope || a.out_dtype != MSPR_F32)
     return false;
+  // MSPR_PREFILL_PERSISTENT=0 (read per call, like the reference's consumer switches) keeps every prefill call on
+  // the split kernel, one workgroup per token: the form to compare the persistent consumer with
+  const char* gate = getenv("MSPR_PREFILL_PERSISTENT");
+  if (gate && gate[0] == '0' && gate[1] == '\0') return false;
   if (a.subst_row || a.subst_from_params || a.pool_rows_dev) return false;
   const int tiles = (a.n_win + kTile - 1) / kTile + (a.n_idx + kTile - 1) / kTile;
   return tiles <= PrefillGeometry::kMaxTiles;
