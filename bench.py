@@ -333,6 +333,16 @@ def bench_ds4_prefill(dev, gen, reps=5):
         "workload": "3844-token chunk, 64 heads x 512, 961 pool rows, top-512, window 128 (float16 operands)",
     }
     out["partial_rope_GBps"] = round(2 * q.numel() * 2 / (out["partial_rope_query_ms"] * 1e-3) / 1e9, 1)
+    # the same chunk deep in a context: every token sees its whole window and all 512 selected rows, the pool is
+    # larger than one L2 (at position 0 half of the ids lie behind the stop position and their tiles are not run)
+    pos_deep = 28000
+    p_deep = (pos_deep + T) // 4
+    comp_deep = torch.randn((1, p_deep, 512), device=dev, generator=gen).to(torch.float16)
+    ids_deep = torch.stack([torch.sort(torch.randperm(p_deep, device=dev, generator=gen)[:512]).values for _ in range(T)])
+    ids_deep = ids_deep[None].to(torch.int32).contiguous()
+    out["indexed_attention_deep_ms"] = timed(lambda: iak.indexed_mixed_attention_prefill_live_f16(
+        q, raw, comp_deep, ids_deep, sinks, pos0=pos_deep, window=128, ratio=4))
+    out["workload_deep"] = f"the same chunk from position {pos_deep}: {p_deep} pool rows, 640 rows per token"
     return out
 
 
