@@ -134,6 +134,13 @@ int mspr_indexer_scores_tiled_live(const void* q, const float* weights, const vo
 /* Scratch bytes for the gathered-attention entry points below. */
 size_t mspr_sparse_attention_workspace_bytes(int batch, int n_heads, int64_t n_keys);
 
+/* Scratch bytes for mspr_indexed_mixed_attention_prefill: the per-range partials of calls that take one workgroup
+ * per token, or the half-precision copy of float32 queries (batch*n_tokens*n_heads*512*2 bytes), whichever is
+ * larger. window_rows is the largest number of ring rows a token attends. No counterpart in the reference
+ * (its kernels allocate through MLX). */
+size_t mspr_indexed_mixed_attention_prefill_workspace_bytes(int q_dtype, int batch, int n_heads, int n_tokens,
+                                                            int window_rows, int top_k);
+
 /* One-token indexed mixed attention over a ring of raw rows plus gathered pool rows, K == V.
  * Replaces indexed_mixed_attention_decode, indexed_attention_kernel.py:1496 (kernel :61-174).
  * q: f32 [n_heads,512] (rounded to half on load); raw_kv: f16 [raw_cap,512];
@@ -157,11 +164,13 @@ int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, const void*
  * 512 contiguous values of q_dtype (f32 rounded to half on load, or f16); raw_kv: f16
  * [batch,raw_cap,512]; comp_kv: f16 [batch,n_comp,512]; topk: int32 [batch,n_tokens,top_k]
  * (top_k may be 0); sinks: f32 [n_heads]; out: f32 with the strides of q.
- * Float16 queries whose slot count fits 22 tiles of 32 (window and ids each rounded up to whole tiles) run on
- * one persistent workgroup per CU that streams consecutive tokens; other calls take one workgroup per token and
- * key range (every call does with MSPR_PREFILL_PERSISTENT=0 in the environment, read per call). The arguments
- * and the workspace size asked for are the same either way.
- * Workspace: mspr_sparse_attention_workspace_bytes(batch*n_tokens, n_heads, min(window or raw_cap, raw_cap) + top_k). */
+ * Calls whose slot count fits 22 tiles of 32 (window and ids each rounded up to whole tiles) run on one
+ * persistent workgroup per CU that streams consecutive tokens; float32 queries are first rounded to half into
+ * the workspace. Other calls take one workgroup per token and key range (every call does with
+ * MSPR_PREFILL_PERSISTENT=0 in the environment, read per call). The arguments and the workspace size asked
+ * for are the same either way.
+ * Workspace: mspr_indexed_mixed_attention_prefill_workspace_bytes(q_dtype, batch, n_heads, n_tokens,
+ * min(window or raw_cap, raw_cap), top_k). */
 int mspr_indexed_mixed_attention_prefill(const void* q, int q_dtype, int batch, int n_heads, int n_tokens,
                                          int64_t q_batch_stride, int64_t q_head_stride,
                                          int64_t q_token_stride, const void* raw_kv, int raw_cap,

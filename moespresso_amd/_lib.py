@@ -50,6 +50,7 @@ SIGNATURES = {
         c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64,
                 c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mspr_sparse_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int64]),
+    "mspr_indexed_mixed_attention_prefill_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "mspr_indexed_mixed_attention_decode": (
         c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_int64,
                 c_int, c_int, c_int, c_void_p, c_void_p, c_size_t, c_void_p]),
@@ -112,6 +113,14 @@ def profile_collect(name: str, max_n: int = 65536) -> list[float]:
 def sparse_attention_workspace(batch: int, n_heads: int, n_keys: int, device) -> torch.Tensor:
     """Scratch tensor for the gathered-attention entry points (split partials)."""
     nbytes = int(lib().mspr_sparse_attention_workspace_bytes(int(batch), int(n_heads), int(n_keys)))
+    return torch.empty((max(nbytes, 16) + 3) // 4, dtype=torch.float32, device=device)
+
+
+def prefill_attention_workspace(q_dtype, batch: int, n_heads: int, n_tokens: int, window_rows: int, top_k: int,
+                                device) -> torch.Tensor:
+    """Scratch tensor for mspr_indexed_mixed_attention_prefill (split partials, or the half copy of float32 queries)."""
+    nbytes = int(lib().mspr_indexed_mixed_attention_prefill_workspace_bytes(
+        DTYPE_CODE[q_dtype], int(batch), int(n_heads), int(n_tokens), int(window_rows), int(top_k)))
     return torch.empty((max(nbytes, 16) + 3) // 4, dtype=torch.float32, device=device)
 
 

@@ -66,15 +66,8 @@ def build(verbose: bool = True) -> str:
     return LIB_PATH
 
 
-def kernel_resources(src: str) -> dict[str, dict[str, int]]:
-    """Registers and scratch of every kernel in one HIP source, from the code object metadata of a device-only
-    compile to assembly: ``{kernel symbol: {"vgprs", "sgprs", "scratch_bytes", "vgpr_spills", "sgpr_spills"}}``.
-
-    The kernels that count their own vector-memory operations (asynchronous tile copies awaited with
-    ``s_waitcnt vmcnt(n)``) rely on the compiler adding none: a register spilled to scratch is one more
-    vector-memory operation in the middle of the count, and its reload drains every copy in flight.
-    """
-    import re
+def device_assembly(src: str) -> str:
+    """gfx950 assembly of one HIP source (device-only compile, nothing runs)."""
     import tempfile
 
     with tempfile.TemporaryDirectory() as tmp:
@@ -83,7 +76,20 @@ def kernel_resources(src: str) -> dict[str, dict[str, int]]:
         proc = subprocess.run(cmd, capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src}:\n{proc.stderr}")
-        text = open(out).read()
+        return open(out).read()
+
+
+def kernel_resources(src: str, text: str | None = None) -> dict[str, dict[str, int]]:
+    """Registers and scratch of every kernel in one HIP source, from the code object metadata of a device-only
+    compile to assembly: ``{kernel symbol: {"vgprs", "sgprs", "scratch_bytes", "vgpr_spills", "sgpr_spills"}}``.
+
+    The kernels that count their own vector-memory operations (asynchronous tile copies awaited with
+    ``s_waitcnt vmcnt(n)``) rely on the compiler adding none: a register spilled to scratch is one more
+    vector-memory operation in the middle of the count, and its reload drains every copy in flight.
+    """
+    import re
+
+    text = device_assembly(src) if text is None else text
     fields = {"vgprs": "vgpr_count", "sgprs": "sgpr_count", "scratch_bytes": "private_segment_fixed_size",
               "vgpr_spills": "vgpr_spill_count", "sgpr_spills": "sgpr_spill_count"}
     kernels: dict[str, dict[str, int]] = {}
@@ -97,6 +103,35 @@ def kernel_resources(src: str) -> dict[str, dict[str, int]]:
             for key, field in fields.items()
         }
     return kernels
+
+
+def kernel_bodies(text: str) -> dict[str, list[str]]:
+    """Instruction lines of every kernel of an assembly text: ``{kernel symbol: [line, ...]}``."""
+    import re
+
+    bodies: dict[str, list[str]] = {}
+    for m in re.finditer(r"^(\w+):[^\n]*\n(.*?)^\s*\.end_amdhsa_kernel", text, flags=re.S | re.M):
+        if ".amdhsa_kernel " + m.group(1) in m.group(2):
+            bodies[m.group(1)] = m.group(2).split(".section")[0].splitlines()
+    return bodies
+
+
+def inline_asm_register_loads(lines: list[str]) -> list[str]:
+    """Memory loads with a register destination that come from inline asm statements (the compiler brackets those
+    with ``;;#ASMSTART`` / ``;;#ASMEND``). The compiler takes the outputs of an asm statement for valid the moment
+    the statement ends, so a load issued that way may see its destination register moved, reused or spilled while
+    the data is still in flight; loads whose destination is LDS write no register and are exempt."""
+    import re
+
+    found, inside = [], False
+    for line in lines:
+        if "#ASMSTART" in line:
+            inside = True
+        elif "#ASMEND" in line:
+            inside = False
+        elif inside and re.search(r"\b(global|buffer|flat|scratch)_load|\bs_(buffer_)?load", line) and "_lds_" not in line:
+            found.append(line.strip())
+    return found
 
 
 if __name__ == "__main__":

@@ -15,4 +15,4 @@ void mspr_set_error(const char* fmt, ...) {
 
 extern "C" const char* mspr_last_error(void) { return g_last_error; }
 
-extern "C" int mspr_abi_version(void) { return 4; }
+extern "C" int mspr_abi_version(void) { return 5; }

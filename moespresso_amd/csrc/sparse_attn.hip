@@ -751,7 +751,17 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_split_kernel(SparseAt
 //
 // Ring: behind barrier C of step s every wave has left the V^T reads of tile s-1, so the copies of tile
 // s+3 go into its buffer; every wave waits for its own copies of tile s+1 before C, so tile s+1 is complete
-// when K.Q^T of it starts. Vector-memory waits count younger loads only, never stores.
+// when K.Q^T of it starts.
+//
+// Vector-memory waits. The tile copies, the id fetches and the cache warm-up of the query rows are asynchronous
+// global -> LDS copies issued through asm: they write no register, so nothing the compiler does with registers
+// can meet a load in flight. A wave counts them as it issues them (`issued`) and remembers the count behind each
+// request (a mark); "this request has landed" is s_waitcnt vmcnt(issued - mark), since a wave's vector-memory
+// operations complete in the order issued. Everything else (query rows, the sink, the output stores) is an
+// ordinary load or store that the compiler sees and waits for itself; the query rows are forced complete at a
+// chosen place by an empty asm statement that names their registers. Operations the count leaves out only make
+// a wait longer, never shorter; the output stores are counted (sixteen per wave) so that the waits of a token's
+// first steps do not cover the stores of the token before it.
 // ---------------------------------------------------------------------------------------------------
 struct PrefillGeometry {
   using G = Geometry<512>;
@@ -772,10 +782,13 @@ struct PrefillGeometry {
   static constexpr int kOffP = kOffVmask + 2 * 32 * 4;               // [2 steps][64 heads][kPPitch]
   static constexpr int kOffTmax = kOffP + 2 * 64 * kPPitch;          // [8 waves][16 heads] float
   static constexpr int kOffL = kOffTmax + kWaves * 16 * 4;           // [8 waves][16 heads] float
-  static constexpr int kOffFlag = kOffL + kWaves * 16 * 4;           // flag[2], stop[2]
-  static constexpr int kOffWarm = kOffFlag + 16;                     // [8 waves][64 lanes] dwords nobody reads
-  static constexpr int kLdsBytes = kOffWarm + kWaves * 256;
-  static_assert(kTileSlots == G::kInstr * 64 && kOffTable % 16 == 0 && kOffP % 16 == 0 && kLdsBytes <= 160 * 1024, "LDS map of the prefill consumer");
+  static constexpr int kOffIds = kOffL + kWaves * 16 * 4;            // [2][512] ids of the unit in preparation
+  static constexpr int kOffFlag = kOffIds + 2 * kThreads * 4;        // flag[2], stop[2]
+  static constexpr int kOffWarm = kOffFlag + 16;                     // [64 lanes] dwords nobody reads (every wave's)
+  static constexpr int kLdsBytes = kOffWarm + 256;
+  static_assert(kTileSlots == G::kInstr * 64 && kOffTable % 16 == 0 && kOffP % 16 == 0 && kOffIds % 16 == 0 &&
+                    kLdsBytes <= 160 * 1024,
+                "LDS map of the prefill consumer");
 };
 
 __device__ __forceinline__ f32x4_t mfma16_f16(u32x4_t a, u32x4_t b, f32x4_t c) {
@@ -783,25 +796,22 @@ __device__ __forceinline__ f32x4_t mfma16_f16(u32x4_t a, u32x4_t b, f32x4_t c) {
                                                 0);
 }
 
-// s_waitcnt vmcnt(n) for a wave-uniform n (the counts that the prefill kernel can ask for; anything else waits
-// for everything), then the LDS wait and the barrier
-__device__ __forceinline__ void wait_vm_dyn_and_barrier(int n) {
+// s_waitcnt vmcnt(n) for a wave-uniform n: at most n of this wave's vector-memory operations stay in flight
+// (a count above the cases waits for everything, which is always allowed)
+#define MSPR_VM_CASE(n) case n: asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); break;
+__device__ __forceinline__ void wait_vm_dyn(int n) {
   switch (n) {
-    case 4: wait_vm_and_barrier<4>(); break;
-    case 5: wait_vm_and_barrier<5>(); break;
-    case 6: wait_vm_and_barrier<6>(); break;
-    case 7: wait_vm_and_barrier<7>(); break;
-    case 8: wait_vm_and_barrier<8>(); break;
-    case 10: wait_vm_and_barrier<10>(); break;
-    case 20: wait_vm_and_barrier<20>(); break;
-    case 21: wait_vm_and_barrier<21>(); break;
-    case 22: wait_vm_and_barrier<22>(); break;
-    case 23: wait_vm_and_barrier<23>(); break;
-    case 38: wait_vm_and_barrier<38>(); break;
-    case 39: wait_vm_and_barrier<39>(); break;
-    default: wait_vm_and_barrier<0>(); break;
+    MSPR_VM_CASE(1) MSPR_VM_CASE(2) MSPR_VM_CASE(3) MSPR_VM_CASE(4) MSPR_VM_CASE(5) MSPR_VM_CASE(6) MSPR_VM_CASE(7)
+    MSPR_VM_CASE(8) MSPR_VM_CASE(9) MSPR_VM_CASE(10) MSPR_VM_CASE(11) MSPR_VM_CASE(12) MSPR_VM_CASE(13)
+    MSPR_VM_CASE(14) MSPR_VM_CASE(15) MSPR_VM_CASE(16) MSPR_VM_CASE(17) MSPR_VM_CASE(18) MSPR_VM_CASE(19)
+    MSPR_VM_CASE(20) MSPR_VM_CASE(21) MSPR_VM_CASE(22) MSPR_VM_CASE(23) MSPR_VM_CASE(24) MSPR_VM_CASE(25)
+    MSPR_VM_CASE(26) MSPR_VM_CASE(27) MSPR_VM_CASE(28) MSPR_VM_CASE(29) MSPR_VM_CASE(30) MSPR_VM_CASE(31)
+    MSPR_VM_CASE(32) MSPR_VM_CASE(33) MSPR_VM_CASE(34) MSPR_VM_CASE(35) MSPR_VM_CASE(36) MSPR_VM_CASE(37)
+    MSPR_VM_CASE(38) MSPR_VM_CASE(39) MSPR_VM_CASE(40)
+    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
   }
 }
+#undef MSPR_VM_CASE
 
 struct PrefillUnit {
   int b, t, hb, seq;
@@ -825,7 +835,7 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // (uniform: what is derived from it stays scalar)
   // O^T = V^T.P^T: wave = (head group of 32, quarter of the output columns), lane = (head n, half g)
   const int hg = wave >> 2;
   const int dh = wave & 3;
@@ -840,6 +850,9 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
   const unsigned char* p_rd = lds + PG::kOffP + (32 * hg + n) * PG::kPPitch + 8 * g;
   const int tmax_rd = (2 * (2 * hg + (n >> 4))) * 16 + (n & 15);  // first of the two blocks that hold head 32 hg + n
   const int k_mine = wave < G::kLastWaves ? G::kPerThread : G::kPerThread - 1;  // copies of this wave per tile
+  // this wave's asynchronous copies, counted as they are issued; a mark is the count right behind a request
+  int issued = 0;
+  int mark_t0 = 0, mark_t1 = 0, mark_t2 = 0, mark_t3 = 0, mark_ids = 0;
 
   const int n_units = a.batch * a.n_hblk;
   const int stride = (int)gridDim.x;
@@ -877,17 +890,30 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     const int nt = m.wt + (stop_pos + kTile - 1) / kTile;
     return nt < PG::kMinTiles ? PG::kMinTiles : nt;
   };
-  // ids of this thread's two table slots (slot ls = tid + 512 j; gathered part starts at slot 32 wt): always two
-  // loads with every lane active, index clamped, so that the count of loads in flight is the same in every wave
-  auto request_ids = [&](const PrefillUnit& m, int (&ids)[2]) {
+  // ids of this thread's two table slots (slot ls = tid + 512 j; gathered part starts at slot 32 wt), fetched
+  // straight into LDS: always two copies with every lane active, index clamped. A wave reads back only what it
+  // fetched itself, so its own wait is all that stands between the request and the read.
+  const int* ids_lds = reinterpret_cast<const int*>(lds + PG::kOffIds);
+  const uint32_t ids_lds_wave = __builtin_amdgcn_readfirstlane(
+      (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, lds + PG::kOffIds + wave * 256));
+  auto request_ids = [&](const PrefillUnit& m) {
     const int32_t* idx_b = a.idx + (int64_t)m.seq * a.idx_batch_stride;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       int gi = tid + kThreads * j - m.wt * kTile;
       gi = gi < 0 ? 0 : (gi >= a.n_idx ? a.n_idx - 1 : gi);
       const int32_t* p = idx_b + gi;
-      asm volatile("global_load_dword %0, %1, off" : "=&v"(ids[j]) : "v"(p) : "memory");
+      // lane i's dword lands at ids_lds[64 wave + 512 j + i] = ids_lds[tid + 512 j]
+      asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(p), "s"(ids_lds_wave + j * (kThreads * 4))
+                   : "memory", "m0");
     }
+    issued += 2;
+    mark_ids = issued;
+  };
+  auto await_ids = [&](int (&ids)[2]) {
+    wait_vm_dyn(issued - mark_ids);
+    ids[0] = ids_lds[tid];
+    ids[1] = ids_lds[tid + kThreads];
   };
   // position of the first id that ends the walk (>= the visible prefix), minimum over the workgroup
   auto scan_stop = [&](const PrefillUnit& m, const int (&ids)[2], int* stop) {
@@ -943,7 +969,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     const int row = P / PG::kSlots, chunk = P % PG::kSlots;
     pk[j] = (P < PG::kTileSlots && chunk < 64) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
   }
-  auto copy_tile = [&](int slot, int tile, int buf) {
+  auto copy_tile = [&](int slot, int tile, int flat) {
+    const int buf = flat & (PG::kBufs - 1);
     const uint64_t* rp = table + slot * PG::kTableSlots + tile * kTile;
     uint64_t src[G::kPerThread];
 #pragma unroll
@@ -957,6 +984,18 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
 #pragma unroll
     for (int j = 0; j < G::kPerThread; j++)
       if (j < G::kPerThread - 1 || wave < G::kLastWaves) async_load_16(src[j], dst_lds + j * (kWaves * 1024));
+    issued += k_mine;
+    mark_t0 = buf == 0 ? issued : mark_t0;
+    mark_t1 = buf == 1 ? issued : mark_t1;
+    mark_t2 = buf == 2 ? issued : mark_t2;
+    mark_t3 = buf == 3 ? issued : mark_t3;
+  };
+  static_assert(PG::kBufs == 4, "ring index by mask");
+  // this wave's copies of flat tile j have landed
+  auto await_tile = [&](int flat) {
+    const int buf = flat & (PG::kBufs - 1);
+    const int mark = buf == 0 ? mark_t0 : (buf == 1 ? mark_t1 : (buf == 2 ? mark_t2 : mark_t3));
+    wait_vm_dyn(issued - mark);
   };
 
   // ---- query operand of a unit: lane (c16 = head of the quarter, kg) holds q[head][32 ks + 8 kg .. +7]
@@ -966,34 +1005,31 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     const int64_t qoff = (int64_t)m.b * a.q_batch_stride + (int64_t)m.t * a.q_token_stride +
                          (int64_t)(head < a.n_heads ? head : 0) * a.q_head_stride + 8 * kg;
     const uint16_t* qp = reinterpret_cast<const uint16_t*>(a.q) + qoff;
+    // (ordinary loads: the compiler knows these registers are in flight until it has waited for them)
 #pragma unroll
-    for (int ks = 0; ks < PG::kQSteps; ks++) {
-      const uint16_t* p = qp + 32 * ks;
-      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(qf[ks]) : "v"(p) : "memory");
-    }
+    for (int ks = 0; ks < PG::kQSteps; ks++) qf[ks] = *reinterpret_cast<const u32x4_t*>(qp + 32 * ks);
   };
   // one dword of every 128-byte line of a unit's query rows (64 rows of 1 KB), requested long before the rows
-  // themselves so that those come out of the L2. The dwords go to LDS nobody reads: a load into a register
-  // that is dead behind the request would land in whatever the register holds by then.
-  const uint32_t warm_lds = __builtin_amdgcn_readfirstlane(
-      (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, lds + PG::kOffWarm + wave * 256));
+  // themselves so that those come out of the L2. The dwords go to LDS nobody reads (the same 256 bytes for
+  // every wave).
+  const uint32_t warm_lds =
+      __builtin_amdgcn_readfirstlane((uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, lds + PG::kOffWarm));
   auto warm_q = [&](const PrefillUnit& m) {
     const int head = m.hb * 64 + (tid >> 3);
     const uint16_t* p = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)m.b * a.q_batch_stride +
                         (int64_t)m.t * a.q_token_stride + (int64_t)(head < a.n_heads ? head : 0) * a.q_head_stride +
                         (tid & 7) * 64;
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" ::"v"(p), "s"(warm_lds) : "memory", "m0");
+    issued += 1;
   };
   static_assert(PG::kQSteps == 16, "the query wait below names sixteen registers");
 #define MSPR_QF_OPERANDS                                                                                             \
   "+v"(qf[0]), "+v"(qf[1]), "+v"(qf[2]), "+v"(qf[3]), "+v"(qf[4]), "+v"(qf[5]), "+v"(qf[6]), "+v"(qf[7]), "+v"(qf[8]), \
       "+v"(qf[9]), "+v"(qf[10]), "+v"(qf[11]), "+v"(qf[12]), "+v"(qf[13]), "+v"(qf[14]), "+v"(qf[15])
-  auto await_q = [&](int newer) {  // at most `newer` younger loads of this wave may stay in flight
-    if (newer == G::kPerThread) asm volatile("s_waitcnt vmcnt(%16)" : MSPR_QF_OPERANDS : "n"(G::kPerThread) : "memory");
-    else if (newer == G::kPerThread - 1)
-      asm volatile("s_waitcnt vmcnt(%16)" : MSPR_QF_OPERANDS : "n"(G::kPerThread - 1) : "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" : MSPR_QF_OPERANDS : : "memory");
-  };
+  // The query rows have to be complete here: the statement uses their registers, so the compiler puts its wait
+  // in front of it (and not in front of their first use in a matrix instruction, behind tile copies that the
+  // wait would then cover too).
+  auto await_q = [&]() { asm volatile("" : MSPR_QF_OPERANDS : : "memory"); };
 #undef MSPR_QF_OPERANDS
   auto mask_q = [&](const PrefillUnit& m) {
     if (m.hb * 64 + 16 * hq + c16 >= a.n_heads) {
@@ -1004,20 +1040,20 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
 
   // ---- first unit: ids, stop position, table, query, first three tiles
   PrefillUnit cur = unit_of(unit);
-  int ids[2];
+  int ids[2] = {-1, -1};
   const bool have_ids = a.n_idx > 0;
-  if (have_ids) request_ids(cur, ids); else ids[0] = ids[1] = -1;
+  if (have_ids) request_ids(cur);
   request_q(cur);
   if (tid == 0) stop_sh[0] = a.n_idx;
   __syncthreads();
   if (have_ids) {
-    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(ids[0]), "+v"(ids[1]) : "n"(PG::kQSteps) : "memory");
+    await_ids(ids);
     scan_stop(cur, ids, &stop_sh[0]);
   }
   __syncthreads();
   int n_cur = tiles_of(cur, stop_sh[0]);
   build_table(cur, 0, ids, stop_sh[0], n_cur);
-  await_q(0);
+  await_q();
   mask_q(cur);
   // sink of this lane's head (a plain load: its wait would drain the tile copies anywhere behind this point)
   float sink_l2;
@@ -1063,13 +1099,12 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
   };
 
   // tile 0 is complete once every wave's copies of it are (the copies of tiles 1 and 2 stay in flight)
-  wait_vm_dyn_and_barrier(2 * k_mine);
+  await_tile(0);
+  lds_barrier();
   f32x4_t sacc = qk_block(kbuf);
 
-  int s = 0;           // tiles done by this workgroup: ring buffer s % 4, flag and P^T slot s & 1
-  int slot = 0;        // table slot of the current unit
-  int prev_extra = 0;  // loads other than tile copies that this wave requested in the step before
-  int stores_behind = 0;  // output stores of the unit before (16 per wave that holds a live head)
+  int s = 0;     // tiles done by this workgroup: ring buffer s % 4, flag and P^T slot s & 1
+  int slot = 0;  // table slot of the current unit
   for (;;) {
     const bool have_next = unit + stride < n_units;
     PrefillUnit nxt = cur;
@@ -1080,31 +1115,16 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     for (int t = 0; t < n_cur; t++, s++) {
       const bool last = t == n_cur - 1;
       // ---- what the next unit needs, at fixed places of this unit's stream
-      int extra = 0;
       if (have_next) {
         if (t == 1 && have_ids) {
-          // (younger loads of this wave: the copies issued behind barrier C of the step before)
-          if (k_mine == G::kPerThread)
-            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(nids[0]), "+v"(nids[1]) : "n"(G::kPerThread) : "memory");
-          else
-            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(nids[0]), "+v"(nids[1]) : "n"(G::kPerThread - 1) : "memory");
+          await_ids(nids);  // (requested a step ago; younger: the copies issued behind barrier C of that step)
           scan_stop(nxt, nids, &stop_sh[slot ^ 1]);
         }
         if (t == 0) {
-          if (have_ids) {
-            request_ids(nxt, nids);
-            extra = 2;
-          }
+          if (have_ids) request_ids(nxt);
           if (tid == 0) stop_sh[slot ^ 1] = a.n_idx;
         }
-        if (t == 2) {
-          warm_q(nxt);
-          extra = 1;
-        }
-        if (last) {  // K.Q^T of this unit's last tile ran in the step before: the query registers are free
-          request_q(nxt);
-          extra = PG::kQSteps;
-        }
+        if (t == 2) warm_q(nxt);
       }
       // ---- softmax weights of this wave's block: head 16 hq + c16, keys 16 kh + 4 kg + i
       float sv[4];
@@ -1125,13 +1145,10 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
         *reinterpret_cast<u32x2_t*>(p_wr_s) = u32x2_t{pack2<KDT>(pw[0], pw[1]), pack2<KDT>(pw[2], pw[3])};
       }
       if (__any(tloc > m_qk + kGrow) && lane == 0) flag[s & 1] = s + 1;
-      // tile s+1 complete behind this barrier: this wave's copies of it are older than everything it has
-      // requested since (the copies of tile s+2, and ids or query rows in this step and the one before)
-      const bool two_ahead = t + 2 < n_cur || have_next;
-      // (the stores of the unit before are younger than the awaited copies in its first two steps; loads and
-      // stores of a wave complete in the order issued)
-      wait_vm_dyn_and_barrier(prev_extra + (two_ahead ? k_mine : 0) + extra + (t < 2 ? stores_behind : 0));  // C
-      prev_extra = extra;
+      // tile s+1 complete behind this barrier: every wave waits for its own copies of it, leaving in flight
+      // what it has issued since (the copies of tile s+2, ids, the warm-up dword, the stores of the unit before)
+      if (!last || have_next) await_tile(s + 1);
+      lds_barrier();  // C
       if (__builtin_amdgcn_readfirstlane(flag[s & 1]) == s + 1) {
         // ---- a key above the common maximum: the waves agree on a new one and write P^T again
         if (kg == 0) tmaxbuf[wave * 16 + c16] = tloc;
@@ -1168,18 +1185,14 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
           la_tile -= n_cur;
           ahead = have_next;
         }
-        if (ahead) copy_tile(la_slot, la_tile, (s + 3) % PG::kBufs);
+        if (ahead) copy_tile(la_slot, la_tile, s + 3);
       }
       if (have_next && t == 1) {
         const int stop_pos = stop_sh[slot ^ 1];
         n_nxt = __builtin_amdgcn_readfirstlane(tiles_of(nxt, stop_pos));
         build_table(nxt, slot ^ 1, nids, stop_pos, n_nxt);
       }
-      if (have_next && last) {
-        await_q(k_mine);  // (younger: the copies issued just above)
-        mask_q(nxt);
-      }
-      // ---- O^T += V^T . P^T of tile s, and S^T of tile s+1
+      // ---- O^T += V^T . P^T of tile s, and S^T of tile s+1 (of the next unit's first tile: behind its query rows)
       const unsigned char* kt = kbuf + (s % PG::kBufs) * G::kTileBytes;
       const unsigned char* p_rd_s = p_rd + (s & 1) * (64 * PG::kPPitch);
       u32x4_t pf[2];
@@ -1200,9 +1213,13 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
           oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
         }
       }
-      if (!last || have_next) sacc = qk_block(kbuf + ((s + 1) % PG::kBufs) * G::kTileBytes);
+      if (!last) sacc = qk_block(kbuf + ((s + 1) % PG::kBufs) * G::kTileBytes);
     }
 
+    // ---- K.Q^T of this unit's last tile ran a step ago, so the query registers are free: the next unit's rows
+    //      are requested here and arrive while this unit's output leaves. Request, wait and first use sit in
+    //      straight-line code, so no path reaches a use of these registers with the loads in flight.
+    if (have_next) request_q(nxt);
     // ---- end of the unit: the denominators meet, sink, normalise, store
     {
       float l_w = l_qk;
@@ -1213,14 +1230,13 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
       const float l_tot = lbuf[tmax_rd] + lbuf[tmax_rd + 16];
       const int head = cur.hb * 64 + hg * 32 + n;
       const bool q_live = head < a.n_heads;
-      stores_behind = __any(q_live) ? 16 : 0;
       const float sink = sink_l2;
       const float m_all = fmaxf(m_pv, sink);
       const float m_safe = m_all == -__builtin_inff() ? 0.0f : m_all;
       const float w = fast_exp2(m_pv - m_safe);
       const float l = l_tot * w + fast_exp2(sink - m_safe);
       const float f = l == 0.0f ? 0.0f : w / l;
-      if (q_live) {
+      auto store_rows = [&]() {
         const int64_t obase = (int64_t)cur.b * a.out_batch_stride + (int64_t)cur.t * a.out_token_stride +
                               (int64_t)head * a.out_head_stride;
 #pragma unroll
@@ -1232,9 +1248,16 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
             const int dim0 = dh * 128 + 32 * mt + 8 * c + 4 * g;
             emit_output<MSPR_F32>(a, r, obase + dim0, dim0);
           }
-      }
+      };
+      // The query rows requested above are forced complete on every path out of this block (also when there is
+      // no next unit: then nothing is in flight and the statement costs nothing), so that the compiler never
+      // sees a path into the tile loop with those loads outstanding.
+      if (q_live) store_rows();
+      await_q();
+      if (__any(q_live)) issued += 16;  // one store per (mt, c) in every wave that holds a live head
     }
     if (!have_next) break;
+    mask_q(nxt);
     unit += stride;
     if (nxt.hb != cur.hb) {  // (more than 64 heads: the wait of this load drains the copies in flight once)
       const int head = nxt.hb * 64 + hg * 32 + n;
@@ -1249,7 +1272,29 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     m_qk = -__builtin_inff();
     m_pv = -__builtin_inff();
     l_qk = 0.0f;
+    // S^T of the unit's first tile (its copies were awaited in the step before)
+    sacc = qk_block(kbuf + (s % PG::kBufs) * G::kTileBytes);
   }
+}
+
+// Float32 query rows of a prefill chunk rounded to half (nearest even, what the consumer's operand load does to a
+// float32 query) into a dense [batch][token][head][512] copy: the persistent consumer keeps the 64 x 512 query
+// block of a unit in registers, which holds half-precision rows only. A thread converts eight values.
+__global__ __launch_bounds__(256) void prefill_q_to_half_kernel(const float* q, int64_t batch_stride, int64_t head_stride,
+                                                                int64_t token_stride, int n_heads, int n_tokens,
+                                                                int64_t n_rows, uint16_t* dst) {
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // (batch, token, head) flattened
+  if (row >= n_rows) return;
+  const int col = (threadIdx.x & 63) * 8;
+  const int64_t bt = row / n_heads;
+  const int head = (int)(row - bt * n_heads);
+  const int64_t b = bt / n_tokens;
+  const int64_t t = bt - b * n_tokens;
+  const float* src = q + b * batch_stride + t * token_stride + (int64_t)head * head_stride + col;
+  const f32x4_t lo = *reinterpret_cast<const f32x4_t*>(src);
+  const f32x4_t hi = *reinterpret_cast<const f32x4_t*>(src + 4);
+  *reinterpret_cast<u32x4_t*>(dst + row * 512 + col) = u32x4_t{pack2<MSPR_F16>(lo.x, lo.y), pack2<MSPR_F16>(lo.z, lo.w),
+                                                              pack2<MSPR_F16>(hi.x, hi.y), pack2<MSPR_F16>(hi.z, hi.w)};
 }
 
 template <int ODT>
@@ -1395,10 +1440,12 @@ int launch_split(const SparseAttnArgs& a, hipStream_t st) {
   return MSPR_OK;
 }
 
-// The persistent prefill consumer takes float16 queries and at most PrefillGeometry::kMaxTiles tiles per token;
-// everything else goes through the split kernel, one workgroup per token.
+// The persistent prefill consumer takes at most PrefillGeometry::kMaxTiles tiles per token (float32 queries go
+// through a half-precision copy in the workspace first); longer slot lists go through the split kernel, one
+// workgroup per token.
 bool prefill_consumer_fits(const SparseAttnArgs& a, int kv_dtype, int k_dim) {
-  if (!a.prefill || kv_dtype != MSPR_F16 || k_dim != 512 || a.q_dtype != MSPR_F16 || a.rope || a.out_dtype != MSPR_F32)
+  if (!a.prefill || kv_dtype != MSPR_F16 || k_dim != 512 || (a.q_dtype != MSPR_F16 && a.q_dtype != MSPR_F32) || a.rope ||
+      a.out_dtype != MSPR_F32)
     return false;
   // MSPR_PREFILL_PERSISTENT=0 (read per call, like the reference's consumer switches) keeps every prefill call on
   // the split kernel, one workgroup per token: the form to compare the persistent consumer with
@@ -1448,7 +1495,30 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
   auto magic = [](int n) -> uint32_t { return n <= 1 ? 0u : (uint32_t)(((uint64_t)1 << 32) / (uint32_t)n); };
   a.inv_hblk = magic(a.n_hblk);
   a.inv_tokens = magic(a.n_tokens);
-  if (prefill_consumer_fits(a, kv_dtype, k_dim)) return launch_prefill_consumer(a, st);
+  if (prefill_consumer_fits(a, kv_dtype, k_dim)) {
+    if (a.q_dtype == MSPR_F32) {
+      // (a.batch counts sequences = batch entries x tokens)
+      const int64_t n_rows = (int64_t)a.batch * a.n_heads;
+      const size_t need = (size_t)n_rows * 512 * sizeof(uint16_t);
+      MSPR_REQUIRE(workspace && workspace_bytes_given >= need,
+                   "sparse attention (prefill): workspace of %zu bytes needed for the half-precision query copy, "
+                   "%zu given",
+                   need, workspace_bytes_given);
+      MSPR_REQUIRE(mspr_aligned(workspace, 16), "sparse attention: workspace must be 16-byte aligned");
+      MSPR_REQUIRE(a.q_head_stride % 4 == 0 && a.q_token_stride % 4 == 0 && a.q_batch_stride % 4 == 0,
+                   "sparse attention (prefill): float32 q strides must be multiples of 4 elements");
+      prefill_q_to_half_kernel<<<dim3((unsigned)((n_rows + 3) / 4)), dim3(256), 0, st>>>(
+          reinterpret_cast<const float*>(a.q), a.q_batch_stride, a.q_head_stride, a.q_token_stride, a.n_heads,
+          a.n_tokens, n_rows, reinterpret_cast<uint16_t*>(workspace));
+      MSPR_CHECK_LAUNCH("sparse attention (prefill, query conversion)");
+      a.q = workspace;
+      a.q_dtype = MSPR_F16;
+      a.q_head_stride = 512;
+      a.q_token_stride = (int64_t)a.n_heads * 512;
+      a.q_batch_stride = (int64_t)a.n_tokens * a.n_heads * 512;
+    }
+    return launch_prefill_consumer(a, st);
+  }
   a.n_splits = choose_splits(a.batch * a.n_hblk, n_keys);
   a.win_per_split = (a.n_win + a.n_splits - 1) / a.n_splits;
   a.idx_per_split = (a.n_idx + a.n_splits - 1) / a.n_splits;
@@ -1487,6 +1557,19 @@ int run_sparse_attention(SparseAttnArgs a, int kv_dtype, int k_dim, void* worksp
 extern "C" size_t mspr_sparse_attention_workspace_bytes(int batch, int n_heads, int64_t n_keys) {
   if (batch < 1 || n_heads < 1 || n_keys < 0) return 0;
   return workspace_bytes(batch, n_heads, n_keys);
+}
+
+extern "C" size_t mspr_indexed_mixed_attention_prefill_workspace_bytes(int q_dtype, int batch, int n_heads,
+                                                                       int n_tokens, int window_rows, int top_k) {
+  if (batch < 1 || n_heads < 1 || n_tokens < 1 || window_rows < 0 || top_k < 0) return 0;
+  // the per-range partials of the split kernel (slot lists too long for the persistent consumer), or the
+  // half-precision copy of float32 queries for the persistent consumer, whichever is larger
+  size_t need = workspace_bytes(batch * n_tokens, n_heads, (int64_t)window_rows + top_k);
+  if (q_dtype == MSPR_F32) {
+    const size_t copy = (size_t)batch * n_tokens * n_heads * 512 * sizeof(uint16_t);
+    if (copy > need) need = copy;
+  }
+  return need;
 }
 
 extern "C" int mspr_indexed_mixed_attention_decode(const float* q, int n_heads, const void* raw_kv, int raw_cap,

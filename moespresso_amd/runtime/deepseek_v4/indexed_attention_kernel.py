@@ -190,7 +190,7 @@ def _run_prefill(q, raw_kv, comp_kv, topk, sinks, *, batch, n_heads, n_tokens, s
     top_k = int(topk.shape[-1])
     out = torch.empty(q.shape, dtype=torch.float32, device=dev)
     max_win = min(int(window), raw_cap) if int(window) != 0 else raw_cap
-    ws = _lib.sparse_attention_workspace(batch * n_tokens, n_heads, max_win + top_k, dev)
+    ws = _lib.prefill_attention_workspace(q.dtype, batch, n_heads, n_tokens, max_win, top_k, dev)
     rc = _lib.lib().mspr_indexed_mixed_attention_prefill(
         _lib.ptr(q), _lib.DTYPE_CODE[q.dtype], batch, n_heads, n_tokens, strides[0], strides[1], strides[2],
         _lib.ptr(raw_kv), raw_cap, _lib.ptr(comp_kv), n_comp, _lib.ptr(topk) if top_k else None, top_k,

@@ -90,23 +90,54 @@ def _oracle_tokens(q, raw, comp, ids, sinks, tokens, *, pos0, window, ratio, raw
     return out
 
 
-def test_prefill_live_f16_at_the_anchor_chunk():
+@pytest.mark.parametrize("q_dtype", [torch.float16, torch.float32])
+def test_prefill_live_at_the_anchor_chunk(q_dtype):
     """The reference's anchor chunk: 3844 tokens, 64 heads, top-512 of the pool, window 128, here from
     position 5000 on a ring deeper than the chunk with a rotated start, and a pool that becomes visible
     while the chunk proceeds (ids ascending; the walk stops at the first invisible one). Sampled tokens
-    against the oracle."""
+    against the oracle; both query types run on the persistent consumer."""
     from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
 
     T, P, pos0, raw_cap, raw_start = 3844, 2300, 5000, 3900, 1234
     rng = np.random.default_rng(2024)
-    q = rng.standard_normal((1, 64, T, 512), dtype=np.float32).astype(np.float16)
+    q = rng.standard_normal((1, 64, T, 512), dtype=np.float32)
+    if q_dtype == torch.float16:
+        q = q.astype(np.float16)
     raw = rng.standard_normal((1, 1, raw_cap, 512), dtype=np.float32).astype(np.float16)
     comp = rng.standard_normal((1, P, 512), dtype=np.float32).astype(np.float16)
     ids = np.stack([np.sort(rng.choice(P, size=512, replace=False)) for _ in range(T)])[None].astype(np.int32)
     sinks = rng.standard_normal((64,), dtype=np.float32)
     kw = dict(pos0=pos0, window=128, ratio=4, raw_start=raw_start)
-    got = iak.indexed_mixed_attention_prefill_live_f16(_t(q), _t(raw), _t(comp), _t(ids), _t(sinks), **kw).cpu().numpy()
+    fn = iak.indexed_mixed_attention_prefill_live_f16 if q_dtype == torch.float16 else \
+        iak.indexed_mixed_attention_prefill_live_f32
+    got = fn(_t(q), _t(raw), _t(comp), _t(ids), _t(sinks), **kw).cpu().numpy()
     tokens = [0, 1, 63, 127, 128, 129, 1000, 1921, 2500, 3000, 3842, 3843]
+    want = _oracle_tokens(q, raw, comp, ids, sinks, tokens, **kw)
+    for t in tokens:
+        np.testing.assert_allclose(got[0, :, t], want[t], rtol=2e-3, atol=2e-3, err_msg=f"token {t}")
+    assert np.isfinite(got).all()
+
+
+@pytest.mark.parametrize("q_dtype", [torch.float16, torch.float32])
+def test_banded_prefill_at_the_anchor_chunk(q_dtype):
+    """The banded route at the anchor chunk: 3844 tokens from position 5000, a band of 128 positions and every
+    pool row visible at ratio 128 (ascending ids over the whole pool, of which a token sees the first
+    (position + 1) / 128). Sampled tokens against the oracle."""
+    from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
+
+    T, pos0, ratio = 3844, 5000, 128
+    P = (pos0 + T) // ratio
+    rng = np.random.default_rng(2025)
+    q = rng.standard_normal((1, 64, T, 512), dtype=np.float32)
+    if q_dtype == torch.float16:
+        q = q.astype(np.float16)
+    raw = rng.standard_normal((1, 1, T, 512), dtype=np.float32).astype(np.float16)
+    comp = rng.standard_normal((1, P, 512), dtype=np.float32).astype(np.float16)
+    ids = np.ascontiguousarray(np.broadcast_to(np.arange(P, dtype=np.int32), (1, T, P)))
+    sinks = rng.standard_normal((64,), dtype=np.float32)
+    kw = dict(pos0=pos0, window=128, ratio=ratio)
+    got = iak.banded_prefill_attention_live(_t(q), _t(raw), _t(comp), _t(ids), _t(sinks), **kw).cpu().numpy()
+    tokens = [0, 1, 119, 120, 127, 128, 1000, 2000, 3715, 3716, 3842, 3843]
     want = _oracle_tokens(q, raw, comp, ids, sinks, tokens, **kw)
     for t in tokens:
         np.testing.assert_allclose(got[0, :, t], want[t], rtol=2e-3, atol=2e-3, err_msg=f"token {t}")
