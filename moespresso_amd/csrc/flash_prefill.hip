@@ -522,7 +522,7 @@ __global__ __launch_bounds__(kThreads, 1) void flash_prefill_kernel(PrefillArgs 
 
 // Float16 tail rows of the quantised-prefix form: key 32 q8_tiles + j for j in [0, tail_rows), the
 // last (past_len % 32) prefix rows dequantised, then the chunk's own rows converted.
-template <int SDT>
+template <int SDT, int ODT>
 __global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, const void* self_k, const void* self_v,
                                                               int self_dtype, uint16_t* tail_k, uint16_t* tail_v,
                                                               int tail_rows, int first_row) {
@@ -552,19 +552,52 @@ __global__ __launch_bounds__(256) void prefill_q8_tail_kernel(PrefillArgs a, con
       vx = load_as_f32<MSPR_BF16>(self_v, off);
     }
   }
-  // float16 staging: values beyond its range saturate instead of becoming infinite (an infinite key or value
-  // turns the whole output row into NaN)
-  kx = __builtin_amdgcn_fmed3f(kx, -65504.0f, 65504.0f);
-  vx = __builtin_amdgcn_fmed3f(vx, -65504.0f, 65504.0f);
-  tail_k[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(kx);
-  tail_v[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(vx);
+  // 16-bit staging: values beyond the range of the staging type saturate instead of becoming infinite (an
+  // infinite key or value turns the whole output row into NaN)
+  if constexpr (ODT == MSPR_F16) {
+    kx = __builtin_amdgcn_fmed3f(kx, -65504.0f, 65504.0f);
+    vx = __builtin_amdgcn_fmed3f(vx, -65504.0f, 65504.0f);
+    tail_k[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(kx);
+    tail_v[(bh * tail_rows + j) * kD + d] = f32_to_f16_bits(vx);
+  } else {
+    constexpr float kBf16Max = 0x1.fep127f;
+    kx = __builtin_amdgcn_fmed3f(kx, -kBf16Max, kBf16Max);
+    vx = __builtin_amdgcn_fmed3f(vx, -kBf16Max, kBf16Max);
+    tail_k[(bh * tail_rows + j) * kD + d] = f32_to_bf16_bits(kx);
+    tail_v[(bh * tail_rows + j) * kD + d] = f32_to_bf16_bits(vx);
+  }
 }
 
 // Prefix rows [0, n_rows) of the quantised cache as float16 rows of the dense K/V buffers (the form taken for
 // long chunks: the attention kernel then reads every tile as a dense one). Same arithmetic as the in-kernel
 // unpacking (float16 code * scale + bias), so both forms attend the same values. A thread converts 16 codes
 // of K and of V; 16 threads a row, 16 rows a workgroup.
+// 16 unsigned 8-bit codes -> 16 bfloat16 values: code * scale + bias in float32 (one fused multiply-add, scale and
+// bias at their float32 values), rounded once
+__device__ __forceinline__ void dequant16_bf16(u32x4_t c, float sc, float bi, u32x4_t& p0, u32x4_t& p1) {
+#pragma unroll
+  for (int w = 0; w < 4; w++) {
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = __builtin_fmaf((float)((c[w] >> (8 * j)) & 0xFFu), sc, bi);
+    const uint32_t lo = pack2<MSPR_BF16>(v[0], v[1]), hi = pack2<MSPR_BF16>(v[2], v[3]);
+    if (w < 2) {
+      p0[2 * w] = lo;
+      p0[2 * w + 1] = hi;
+    } else {
+      p1[2 * (w - 2)] = lo;
+      p1[2 * (w - 2) + 1] = hi;
+    }
+  }
+}
 template <int SDT>
+__device__ __forceinline__ float sb_to_f32(uint32_t bits) {
+  if constexpr (SDT == MSPR_F32) return __builtin_bit_cast(float, bits);
+  else if constexpr (SDT == MSPR_F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+  else return __builtin_bit_cast(float, bits << 16);
+}
+
+template <int SDT, int ODT>
 __global__ __launch_bounds__(256) void prefill_q8_dequant_kernel(PrefillArgs a, uint16_t* out_k, uint16_t* out_v,
                                                                  int64_t n_rows, int64_t out_rows) {
   const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
@@ -583,10 +616,12 @@ __global__ __launch_bounds__(256) void prefill_q8_dequant_kernel(PrefillArgs a, 
   }
   u32x4_t p0, p1;
   const int64_t dst = (bh * out_rows + row) * kD + 16 * pp;
-  dequant16(rk, sb_to_h2<SDT>(rs[0]), sb_to_h2<SDT>(rs[1]), p0, p1);
+  if constexpr (ODT == MSPR_F16) dequant16(rk, sb_to_h2<SDT>(rs[0]), sb_to_h2<SDT>(rs[1]), p0, p1);
+  else dequant16_bf16(rk, sb_to_f32<SDT>(rs[0]), sb_to_f32<SDT>(rs[1]), p0, p1);
   *reinterpret_cast<u32x4_t*>(out_k + dst) = p0;
   *reinterpret_cast<u32x4_t*>(out_k + dst + 8) = p1;
-  dequant16(rv, sb_to_h2<SDT>(rs[2]), sb_to_h2<SDT>(rs[3]), p0, p1);
+  if constexpr (ODT == MSPR_F16) dequant16(rv, sb_to_h2<SDT>(rs[2]), sb_to_h2<SDT>(rs[3]), p0, p1);
+  else dequant16_bf16(rv, sb_to_f32<SDT>(rs[2]), sb_to_f32<SDT>(rs[3]), p0, p1);
   *reinterpret_cast<u32x4_t*>(out_v + dst) = p0;
   *reinterpret_cast<u32x4_t*>(out_v + dst + 8) = p1;
 }
@@ -835,20 +870,40 @@ extern "C" int mspr_sdpa_fa_prefill_q8(const void* queries, const void* pk_wq, c
   // rows of the dense buffers: prefix rows not left to the attention kernel, then the chunk's own rows
   const int64_t dq_rows = q8_tiles == 0 ? past_len : 0;  // converted 16 codes at a time
   const int first_row = (int)dq_rows;                   // the rest element by element (at most 31 prefix rows + chunk)
+#ifndef MSPR_Q8_LONG_BF16
+#define MSPR_Q8_LONG_BF16 1
+#endif
+  // Long chunks (prefix converted beforehand) stage K/V and the queries as bfloat16 and run the bfloat16 matrix
+  // instructions: the device holds a higher clock under them than under the float16 ones, and the 8-bit codes
+  // leave the rounding of the staging type (2^-9 of a value) below their own step. Short chunks unpack the
+  // prefix inside the attention kernel with packed float16 arithmetic and stay float16 throughout.
+  const bool bf16_staging = MSPR_Q8_LONG_BF16 && q_len >= 1024;  // (then q8_tiles == 0)
+#define MSPR_LAUNCH_BY_SB(KERNEL, GRID, ...)                                                          \
+  do {                                                                                                \
+    if (bf16_staging) {                                                                               \
+      if (sb_dtype == MSPR_F32) KERNEL<MSPR_F32, MSPR_BF16><<<GRID, 256, 0, st>>>(__VA_ARGS__);        \
+      else if (sb_dtype == MSPR_F16) KERNEL<MSPR_F16, MSPR_BF16><<<GRID, 256, 0, st>>>(__VA_ARGS__);   \
+      else KERNEL<MSPR_BF16, MSPR_BF16><<<GRID, 256, 0, st>>>(__VA_ARGS__);                            \
+    } else {                                                                                          \
+      if (sb_dtype == MSPR_F32) KERNEL<MSPR_F32, MSPR_F16><<<GRID, 256, 0, st>>>(__VA_ARGS__);         \
+      else if (sb_dtype == MSPR_F16) KERNEL<MSPR_F16, MSPR_F16><<<GRID, 256, 0, st>>>(__VA_ARGS__);    \
+      else KERNEL<MSPR_BF16, MSPR_F16><<<GRID, 256, 0, st>>>(__VA_ARGS__);                             \
+    }                                                                                                 \
+  } while (0)
   if (dq_rows > 0) {
     dim3 dgrid((unsigned)((dq_rows + 15) / 16), (unsigned)n_kv_heads, (unsigned)batch);
-    if (sb_dtype == MSPR_F32) prefill_q8_dequant_kernel<MSPR_F32><<<dgrid, 256, 0, st>>>(a, tail_k, tail_v, dq_rows, tail_rows);
-    else if (sb_dtype == MSPR_F16) prefill_q8_dequant_kernel<MSPR_F16><<<dgrid, 256, 0, st>>>(a, tail_k, tail_v, dq_rows, tail_rows);
-    else prefill_q8_dequant_kernel<MSPR_BF16><<<dgrid, 256, 0, st>>>(a, tail_k, tail_v, dq_rows, tail_rows);
+    MSPR_LAUNCH_BY_SB(prefill_q8_dequant_kernel, dgrid, a, tail_k, tail_v, dq_rows, tail_rows);
     MSPR_CHECK_LAUNCH("sdpa_fa_prefill_q8 (prefix rows)");
   }
   dim3 tgrid((unsigned)(tail_rows - first_row), (unsigned)n_kv_heads, (unsigned)batch);
-  if (sb_dtype == MSPR_F32) prefill_q8_tail_kernel<MSPR_F32><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows, first_row);
-  else if (sb_dtype == MSPR_F16) prefill_q8_tail_kernel<MSPR_F16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows, first_row);
-  else prefill_q8_tail_kernel<MSPR_BF16><<<tgrid, 256, 0, st>>>(a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows, first_row);
+  MSPR_LAUNCH_BY_SB(prefill_q8_tail_kernel, tgrid, a, self_k, self_v, self_dtype, tail_k, tail_v, tail_rows, first_row);
+#undef MSPR_LAUNCH_BY_SB
   MSPR_CHECK_LAUNCH("sdpa_fa_prefill_q8 (tail rows)");
   // (prefix converted beforehand: the dense kernel, with float32 queries and output)
-  if (q8_tiles == 0) return prefill_launch<MSPR_F16, false, MSPR_F32, true>(a, st);
+  if (q8_tiles == 0) {
+    if (bf16_staging) return prefill_launch<MSPR_BF16, false, MSPR_F32, true>(a, st);
+    return prefill_launch<MSPR_F16, false, MSPR_F32, true>(a, st);
+  }
   if (sb_dtype == MSPR_F32) return prefill_launch<MSPR_F16, true, MSPR_F32>(a, st);
   if (sb_dtype == MSPR_F16) return prefill_launch<MSPR_F16, true, MSPR_F16>(a, st);
   return prefill_launch<MSPR_F16, true, MSPR_BF16>(a, st);

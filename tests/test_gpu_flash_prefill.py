@@ -154,7 +154,8 @@ def test_sdpa_fa_prefill_q8_matches_oracle(past, L, sb_dtype, self_dtype):
     want = qwen.causal_prefill_attention(q, k_all, v_all, scale, past=past)
     err = np.abs(got.cpu().numpy() - want).max()
     assert err < 1e-2, err
-    # observed accuracy is far inside the bar: float16 staging of exactly representable code values
+    # observed accuracy is far inside the bar: 16-bit staging (float16 next to a prefix unpacked in the kernel,
+    # bfloat16 for chunks of 1024 queries and more) of values of magnitude 0.1
     assert err < 2e-3, err
 
 

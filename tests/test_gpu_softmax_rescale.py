@@ -286,9 +286,13 @@ def test_sdpa_fa_prefill_q8_ramp(past, L):
                                     _t(v[:, :, past:]), scale, bq=32, bk=16, stage=2).cpu().numpy()
     assert np.isfinite(got).all()
     assert _min_tile_growth(q[0, 0], k_all[0, 0], scale) > 8.0
-    # the kernel stages queries and the chunk's rows as float16
-    want = qwen.causal_prefill_attention(ds4.round_f16(q), np.concatenate(
-        [k_all[:, :, :past], ds4.round_f16(k_all[:, :, past:])], axis=2), np.concatenate(
-        [v_all[:, :, :past], ds4.round_f16(v_all[:, :, past:])], axis=2), scale, past=past)
+    # the kernel stages the queries and the chunk's own rows in 16 bits: float16 next to a prefix that it unpacks
+    # itself, bfloat16 (prefix included) for chunks of 1024 queries and more, whose prefix is converted beforehand
+    stage = ds4.round_bf16 if L >= 1024 else ds4.round_f16
+    if L >= 1024:
+        k_all, v_all = stage(k_all), stage(v_all)
+    want = qwen.causal_prefill_attention(stage(q), np.concatenate(
+        [k_all[:, :, :past], stage(k_all[:, :, past:])], axis=2), np.concatenate(
+        [v_all[:, :, :past], stage(v_all[:, :, past:])], axis=2), scale, past=past)
     err = np.abs(got - want).max()
     assert err < 1e-2, err
