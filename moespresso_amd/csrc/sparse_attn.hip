@@ -154,6 +154,11 @@ constexpr int kQSame = -1;
 // zeros instead of being predicated off.
 __device__ __attribute__((aligned(16))) const unsigned char g_zero_row[1280] = {0};
 
+// Where the prefill consumer's lanes without a head (a block of fewer than 64 heads) put their output stores, so
+// that the store instructions run with every lane active and the same count in every wave: 512 floats per lane
+// position, never read.
+__device__ __attribute__((aligned(16))) float g_store_sink[64 * 512];
+
 #define MSPR_GLB_PTR(T, p) ((__attribute__((address_space(1))) T*)(p))
 
 // Wait until at most N of this wave's vector-memory operations are outstanding and all of its LDS
@@ -1098,6 +1103,30 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     return se + so;
   };
 
+  // O^T += V^T . P^T of flat tile s (P^T of the step is in LDS behind barrier C)
+  auto pv_tile = [&](int s) {
+    const unsigned char* kt = kbuf + (s % PG::kBufs) * G::kTileBytes;
+    const unsigned char* p_rd_s = p_rd + (s & 1) * (64 * PG::kPPitch);
+    u32x4_t pf[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(p_rd_s + 32 * ks);
+      const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(p_rd_s + 32 * ks + 16);
+      pf[ks] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+      for (int mt = 0; mt < 4; mt++) {
+        const unsigned char* base = kt + tr_off + (16 * ks) * PG::kPitch + mt * 64;
+        s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base));
+        s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base + 8 * PG::kPitch));
+        u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
+        oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
+      }
+    }
+  };
+
   // tile 0 is complete once every wave's copies of it are (the copies of tiles 1 and 2 stay in flight)
   await_tile(0);
   lds_barrier();
@@ -1192,34 +1221,19 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
         n_nxt = __builtin_amdgcn_readfirstlane(tiles_of(nxt, stop_pos));
         build_table(nxt, slot ^ 1, nids, stop_pos, n_nxt);
       }
-      // ---- O^T += V^T . P^T of tile s, and S^T of tile s+1 (of the next unit's first tile: behind its query rows)
-      const unsigned char* kt = kbuf + (s % PG::kBufs) * G::kTileBytes;
-      const unsigned char* p_rd_s = p_rd + (s & 1) * (64 * PG::kPPitch);
-      u32x4_t pf[2];
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-        const u32x2_t lo = *reinterpret_cast<const u32x2_t*>(p_rd_s + 32 * ks);
-        const u32x2_t hi = *reinterpret_cast<const u32x2_t*>(p_rd_s + 32 * ks + 16);
-        pf[ks] = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+      // ---- O^T += V^T . P^T of tile s, and S^T of tile s+1. (The unit's last tile: behind the loop, with the
+      //      request for the next unit's query rows in front of it.)
+      if (!last) {
+        pv_tile(s);
+        sacc = qk_block(kbuf + ((s + 1) % PG::kBufs) * G::kTileBytes);
       }
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-#pragma unroll
-        for (int mt = 0; mt < 4; mt++) {
-          const unsigned char* base = kt + tr_off + (16 * ks) * PG::kPitch + mt * 64;
-          s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base));
-          s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(MSPR_LDS_PTR(s16x4_t, base + 8 * PG::kPitch));
-          u32x2_t lo2 = __builtin_bit_cast(u32x2_t, lo), hi2 = __builtin_bit_cast(u32x2_t, hi);
-          oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
-        }
-      }
-      if (!last) sacc = qk_block(kbuf + ((s + 1) % PG::kBufs) * G::kTileBytes);
     }
 
     // ---- K.Q^T of this unit's last tile ran a step ago, so the query registers are free: the next unit's rows
     //      are requested here and arrive while this unit's output leaves. Request, wait and first use sit in
     //      straight-line code, so no path reaches a use of these registers with the loads in flight.
     if (have_next) request_q(nxt);
+    pv_tile(s - 1);
     // ---- end of the unit: the denominators meet, sink, normalise, store
     {
       float l_w = l_qk;
@@ -1236,25 +1250,26 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
       const float w = fast_exp2(m_pv - m_safe);
       const float l = l_tot * w + fast_exp2(sink - m_safe);
       const float f = l == 0.0f ? 0.0f : w / l;
-      auto store_rows = [&]() {
-        const int64_t obase = (int64_t)cur.b * a.out_batch_stride + (int64_t)cur.t * a.out_token_stride +
-                              (int64_t)head * a.out_head_stride;
+      // Sixteen stores per wave, every lane active (a lane without a head stores into g_store_sink), in straight
+      // line behind the query request: the compiler's wait for the query rows then leaves exactly these stores in
+      // flight (it counts what it issued itself), and the wave's own count of them below is exact.
+      float* orow = q_live ? reinterpret_cast<float*>(a.out) + ((int64_t)cur.b * a.out_batch_stride +
+                                                                 (int64_t)cur.t * a.out_token_stride +
+                                                                 (int64_t)head * a.out_head_stride)
+                           : &g_store_sink[lane * 512];
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++)
+      for (int mt = 0; mt < 4; mt++)
 #pragma unroll
-          for (int c = 0; c < 4; c++) {
-            const float r[4] = {oacc[mt][4 * c] * f, oacc[mt][4 * c + 1] * f, oacc[mt][4 * c + 2] * f,
-                                oacc[mt][4 * c + 3] * f};
-            const int dim0 = dh * 128 + 32 * mt + 8 * c + 4 * g;
-            emit_output<MSPR_F32>(a, r, obase + dim0, dim0);
-          }
-      };
+        for (int c = 0; c < 4; c++) {
+          const int dim0 = dh * 128 + 32 * mt + 8 * c + 4 * g;
+          *reinterpret_cast<f32x4_t*>(orow + dim0) = f32x4_t{oacc[mt][4 * c] * f, oacc[mt][4 * c + 1] * f,
+                                                             oacc[mt][4 * c + 2] * f, oacc[mt][4 * c + 3] * f};
+        }
       // The query rows requested above are forced complete on every path out of this block (also when there is
       // no next unit: then nothing is in flight and the statement costs nothing), so that the compiler never
       // sees a path into the tile loop with those loads outstanding.
-      if (q_live) store_rows();
       await_q();
-      if (__any(q_live)) issued += 16;  // one store per (mt, c) in every wave that holds a live head
+      issued += 16;
     }
     if (!have_next) break;
     mask_q(nxt);
