@@ -15,7 +15,8 @@ the streamed rows between steps.
 
 Prints ONE JSON line (see README of the driver contract): metric/value plus `roofline` for the
 dominant kernel (GPU-side duration from HIP events around that kernel on its launch stream) and
-`cpu_baseline` (the NumPy oracle on a bounded sample, on this host's cores).
+`cpu_baseline` (a threaded torch restatement of the same layer, pinned against the NumPy oracle by the
+CPU tests, on a bounded sample on this host's cores; the float64 NumPy oracle itself is timed beside it).
 """
 
 from __future__ import annotations
@@ -35,12 +36,64 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 COUNTERS_FILE = os.path.join(ROOT, "profiles", "bench_sparse_decode_layer_hbm_counters.txt")
+TRACE_FILE = os.path.join(ROOT, "profiles", "bench_all_kernels_kernel_trace_stats.txt")
+SPLIT_KERNEL_SOURCE = os.path.join(ROOT, "moespresso_amd", "csrc", "sparse_attn.hip")
+
+
+def host_threads() -> int:
+    """Threads the CPU legs use: the host's cores, at most 16 (the CPU share of a one-GPU box)."""
+    return min(16, os.cpu_count() or 1)
+
+
+def source_sha256(path: str = SPLIT_KERNEL_SOURCE) -> str | None:
+    import hashlib
+
+    try:
+        with open(path, "rb") as f:
+            return hashlib.sha256(f.read()).hexdigest()
+    except OSError:
+        return None
+
+
+def profile_is_current(path: str) -> bool:
+    """A committed rocprofv3 summary records the SHA-256 of the kernel source it was taken from (a line
+    `source_sha256 sparse_attn.hip <hex>`); figures from it are reported only while that source is unchanged."""
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("source_sha256 sparse_attn.hip"):
+                    return line.split()[-1] == source_sha256()
+    except OSError:
+        pass
+    return False
+
+
+def traced_kernel_us(kernel_prefix: str, workgroups: str):
+    """Average duration (us) of one kernel and launch shape (`workgroups` as "256x1x1") in the committed
+    `rocprofv3 --kernel-trace --stats` summary of this benchmark (graph-replayed launches: no event records around
+    the kernel), or None."""
+    import re
+
+    if not profile_is_current(TRACE_FILE):
+        return None
+    row = re.compile(r"^(?P<name>.+?)\s+(?P<wg>\d+x\d+x\d+)\s+\d+\s+\d+\s+(?P<avg>[\d.]+)\s+[\d.]+\s+[\d.]+\s*$")
+    try:
+        with open(TRACE_FILE) as f:
+            for line in f:
+                m = row.match(line)
+                if m and m.group("name").startswith(kernel_prefix) and m.group("wg") == workgroups:
+                    return float(m.group("avg"))
+    except (OSError, ValueError):
+        pass
+    return None
 
 
 def measured_traffic_bytes(kernel_prefix: str, workgroups: int):
     """HBM bytes per launch of one kernel as the committed rocprofv3 counter summary reports them (FETCH_SIZE +
     WRITE_SIZE, each scaled by the same counter's reading for a copy kernel of known size); None when the
     summary does not hold that launch shape."""
+    if not profile_is_current(COUNTERS_FILE):
+        return None
     try:
         with open(COUNTERS_FILE) as f:
             for line in f:
@@ -75,6 +128,47 @@ def make_set(batch: int, dev, gen):
     return dict(qi=qi, keys=keys, kscale=kscale, w=w, q=q, kv=kv)
 
 
+def cpu_baseline_torch(seconds_budget: float = 10.0, threads: int | None = None):
+    """The torch restatement of the layer (oracle/ds4_torch.py, float32, threaded) on one sequence of the same
+    step, scaled to the 16-sequence layer."""
+    from oracle import ds4_torch
+
+    cores = host_threads() if threads is None else threads
+    before = torch.get_num_threads()
+    torch.set_num_threads(cores)
+    try:
+        g = torch.Generator().manual_seed(0)
+        qi = torch.randn((N_IDX_HEADS, IDX_DIM), generator=g).to(torch.bfloat16).float()
+        k32 = torch.randn((N_KEYS, IDX_DIM), generator=g)
+        kscale = k32.abs().amax(dim=-1) / 448.0
+        codes = (k32 / kscale[:, None]).to(torch.float8_e4m3fn).view(torch.uint8)
+        w = torch.rand((N_IDX_HEADS,), generator=g)
+        q = torch.randn((N_HEADS, K_DIM), generator=g).to(torch.bfloat16).float()
+        kv = torch.randn((N_TOKENS, K_DIM), generator=g).to(torch.bfloat16)
+
+        def step():
+            return ds4_torch.decode_layer(qi, codes, kscale, w, q, kv, topk=TOPK, window=WINDOW, scale=K_DIM ** -0.5)
+
+        step()
+        t0 = time.perf_counter()
+        reps = 0
+        while reps < 200 and (time.perf_counter() - t0) < seconds_budget:
+            step()
+            reps += 1
+        per_seq = (time.perf_counter() - t0) / max(reps, 1)
+    finally:
+        torch.set_num_threads(before)
+    return {
+        "value": round(per_seq * 16 * 1e6, 1),
+        "unit": "us/layer",
+        "cores": cores,
+        "host_cpus": os.cpu_count(),
+        "kind": "port",
+        "sample": f"{reps} repeats of one sequence (1/16 of the layer: 32768-key indexer + top-2048 + 2176-row "
+                  f"MLA decode), torch float32 restatement of the layer with {cores} threads, scaled x16",
+    }
+
+
 def cpu_baseline(seconds_budget: float = 10.0, threads: int | None = None):
     """The NumPy oracle on one sequence of the same step; scaled to the 16-sequence layer."""
     from oracle import ds4
@@ -83,7 +177,7 @@ def cpu_baseline(seconds_budget: float = 10.0, threads: int | None = None):
         from threadpoolctl import threadpool_limits
     except Exception:  # pragma: no cover
         threadpool_limits = None
-    cores = min(16, os.cpu_count() or 1) if threads is None else threads
+    cores = host_threads() if threads is None else threads
     rng = np.random.default_rng(0)
     qi = ds4.round_bf16(rng.standard_normal((1, N_IDX_HEADS, IDX_DIM), dtype=np.float32))
     k32 = rng.standard_normal((1, N_KEYS, IDX_DIM), dtype=np.float32)
@@ -118,7 +212,8 @@ def cpu_baseline(seconds_budget: float = 10.0, threads: int | None = None):
         "cores": cores,
         "kind": "port",
         "sample": f"{reps} repeats of one sequence (1/16 of the layer: 32768-key indexer + top-2048 + 2176-row "
-                  f"MLA decode), NumPy oracle with {cores} BLAS threads, scaled x16",
+                  f"MLA decode), float64 NumPy oracle with {cores} BLAS threads (its time is the float64 score "
+                  f"sum and the selection, which no BLAS call covers), scaled x16",
     }
 
 
@@ -132,7 +227,7 @@ def cpu_other_configs():
         from threadpoolctl import threadpool_limits
     except Exception:  # pragma: no cover
         threadpool_limits = None
-    cores = min(16, os.cpu_count() or 1)
+    cores = host_threads()
     rng = np.random.default_rng(0)
     out = {}
     ctx = threadpool_limits(limits=cores) if threadpool_limits else None
@@ -189,7 +284,7 @@ def cpu_config1():
     t0 = time.perf_counter()
     for _ in range(20):
         qwen.gqa_decode_attention(q, k, v, 128 ** -0.5).astype(np.float16)
-    return {"us": round((time.perf_counter() - t0) / 20 * 1e6, 1), "kind": "port", "cores": min(16, os.cpu_count() or 1),
+    return {"us": round((time.perf_counter() - t0) / 20 * 1e6, 1), "kind": "port", "cores": 1,
             "workload": "dense GQA decode, 8q/1kv heads, D=128, 4096 fp16 keys (BASELINE config 1), NumPy float64"}
 
 
@@ -255,7 +350,8 @@ def bench_prefill_q8(dev, gen, reps=6, warmup=10):
     tf = flops / (ms * 1e-3) / 1e12
     return {"ms": round(ms, 4), "attention_kernel_ms": round(kernel_ms, 4), "TFLOPs": round(tf, 1),
             "frac": round(tf / 2500.0, 4),
-            "workload": "sdpa_fa_prefill_q8: 4096 new x 32768-token affine 8-bit prefix, float32 queries, float16 MFMA"}
+            "workload": "sdpa_fa_prefill_q8: 4096 new x 32768-token affine 8-bit prefix, float32 queries; prefix converted to "
+                        "bfloat16 rows first, then the bfloat16 MFMA kernel"}
 
 
 def bench_q8_decode(dev, gen, reps=40):
@@ -290,6 +386,33 @@ def bench_q8_decode(dev, gen, reps=40):
                         "frac_of_8TBps": round(nbytes / ((split + merge) * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
         del sets
     out["workload"] = "GQA decode, 16q/2kv heads, D=256, 37000-token int8+f16/32 cache (BASELINE config 3)"
+    # the reference's own decode callable at the same depth: affine 8-bit cache (group 64, bfloat16 scales and
+    # biases as served), float32 queries, batch 1 (runtime/qwen/full_attention.py:323-335 call site)
+    sets = []
+    for _ in range(4):
+        k = kquant.quantize(torch.randn((1, 2, N, 256), device=dev, generator=gen))
+        v = kquant.quantize(torch.randn((1, 2, N, 256), device=dev, generator=gen))
+        k = (k[0], k[1].to(torch.bfloat16), k[2].to(torch.bfloat16))
+        v = (v[0], v[1].to(torch.bfloat16), v[2].to(torch.bfloat16))
+        sets.append((torch.randn((1, 16, 1, 256), device=dev, generator=gen), *k, *v))
+    ws = _lib.q8_decode_workspace(1, 2, N, dev)
+    for s_ in sets:
+        kquant.sdpa_decode_q8(*s_, 256 ** -0.5, workspace=ws)
+    torch.cuda.synchronize()
+    _lib.profile_enable("q8_decode", "q8_merge")
+    for i in range(reps):
+        kquant.sdpa_decode_q8(*sets[i % 4], 256 ** -0.5, workspace=ws)
+    torch.cuda.synchronize()
+    split = float(np.mean(_lib.profile_collect("q8_decode"))) * 1e3
+    merge = float(np.mean(_lib.profile_collect("q8_merge"))) * 1e3
+    _lib.profile_enable()
+    nbytes = N * 2 * 2 * (256 + 16) + 16 * 256 * 8
+    out["affine_sdpa_decode_q8_B1"] = {
+        "split_us": round(split, 2), "merge_us": round(merge, 2),
+        "GBps": round(nbytes / ((split + merge) * 1e-6) / 1e9, 1),
+        "frac_of_8TBps": round(nbytes / ((split + merge) * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+        "workload": "sdpa_decode_q8: affine 8-bit cache (group 64, bfloat16 scales/biases), float32 queries, "
+                    "16q/2kv heads, 37000 keys, batch 1"}
     return out
 
 
@@ -343,6 +466,19 @@ def bench_ds4_prefill(dev, gen, reps=5):
     out["indexed_attention_deep_ms"] = timed(lambda: iak.indexed_mixed_attention_prefill_live_f16(
         q, raw, comp_deep, ids_deep, sinks, pos0=pos_deep, window=128, ratio=4))
     out["workload_deep"] = f"the same chunk from position {pos_deep}: {p_deep} pool rows, 640 rows per token"
+    # the other two forms of the consumer at the same chunk: float32 queries (converted to half into the workspace,
+    # then the same kernel) and the banded route (band of 128 positions + every visible pool row at ratio 128)
+    q32 = q.float()
+    out["indexed_attention_f32_queries_ms"] = timed(lambda: iak.indexed_mixed_attention_prefill_live_f32(
+        q32, raw, comp, ids, sinks, pos0=0, window=128, ratio=4))
+    out["indexed_attention_f32_queries_deep_ms"] = timed(lambda: iak.indexed_mixed_attention_prefill_live_f32(
+        q32, raw, comp_deep, ids_deep, sinks, pos0=pos_deep, window=128, ratio=4))
+    p_band = (pos_deep + T) // 128
+    comp_band = torch.randn((1, p_band, 512), device=dev, generator=gen).to(torch.float16)
+    ids_band = torch.arange(p_band, device=dev, dtype=torch.int32).expand(1, T, p_band).contiguous()
+    out["banded_attention_deep_ms"] = timed(lambda: iak.banded_prefill_attention_live(
+        q, raw, comp_band, ids_band, sinks, pos0=pos_deep, window=128, ratio=128))
+    out["workload_banded"] = f"banded route from position {pos_deep}: band 128, {p_band} pool rows at ratio 128, float16 queries"
     return out
 
 
@@ -482,6 +618,9 @@ def main() -> int:
         "traffic": measured_traffic_bytes("sparse_attn_split_kernel<2, 576", B * 16) if B == 16 else None,
         "algorithmic_bytes_per_launch": MLA_BYTES_PER_SEQ * B,
         "kernel_us": round(split_us, 2),
+        # the same kernel in the committed kernel trace of this benchmark (graph replays, no event records around
+        # the launch: events add about 1.5 us); null when the kernel source has changed since the trace was taken
+        "kernel_us_traced": traced_kernel_us("sparse_attn_split_kernel<2, 576", f"{B * 16}x1x1"),
         # the whole operator (split + merge launches) against the same algorithmic bytes
         "operator_us": round(operator_us, 2),
         "operator_frac": round(MLA_BYTES_PER_SEQ * B / (operator_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
@@ -522,7 +661,8 @@ def main() -> int:
         "ds4_prefill": None if args.headline_only else guarded(bench_ds4_prefill, dev, gen),
         "cpu_config1": None if args.no_cpu_baseline else guarded(cpu_config1),
         "cpu_configs_2_3": None if args.no_cpu_baseline else guarded(cpu_other_configs),
-        "cpu_baseline_1thread": None if args.no_cpu_baseline else guarded(cpu_baseline, seconds_budget=6.0, threads=1),
+        "cpu_baseline_numpy_oracle": None if args.no_cpu_baseline else guarded(cpu_baseline, seconds_budget=6.0),
+        "cpu_baseline_1thread": None if args.no_cpu_baseline else guarded(cpu_baseline_torch, seconds_budget=5.0, threads=1),
         "indexer_fp8_GBps": round(IDX_BYTES_PER_SEQ * B / (kernel_us["indexer_fp8"] * 1e-6) / 1e9, 1),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
         "buffer_sets": R,
@@ -553,7 +693,7 @@ def main() -> int:
             "context": N_TOKENS,
         },
         "roofline": roofline,
-        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline(),
+        "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_torch(),
         "extras": extras,
     }
     print(json.dumps(line))

@@ -623,3 +623,43 @@ def test_fused_decode_prep_all_tie_integer_and_row_parts():
     want = np.stack([x[:, 0] * np.cos(ang) - x[:, 1] * np.sin(ang), x[:, 0] * np.sin(ang) + x[:, 1] * np.cos(ang)], 1)
     np.testing.assert_allclose(row[448:].astype(np.float64), want.reshape(-1), rtol=0, atol=2e-3)
     assert np.abs(row[448:].astype(np.float64) - kv[448:].astype(np.float64)).max() > 0.05    # it did rotate
+
+
+def test_torch_restatement_of_the_decode_layer_matches_the_numpy_oracle():
+    """oracle/ds4_torch.py (the threaded CPU baseline that bench.py times) against the float64 NumPy oracle on a
+    reduced layer: scores to float32 accuracy, the selected set exactly (including a block of tied scores, which
+    go to the lower rows), the attention output to 1e-5."""
+    import torch
+
+    from oracle import ds4_torch
+
+    rng = np.random.default_rng(12)
+    H, N, TOPK, WIN, NT = 64, 2048, 128, 32, 8192
+    qi = ds4.round_bf16(rng.standard_normal((1, H, 128), dtype=np.float32))
+    k32 = rng.standard_normal((1, N, 128), dtype=np.float32)
+    k32[0, 700:716] = k32[0, 700]                      # sixteen identical keys: tied scores
+    ks = (np.abs(k32).max(-1) / 448).astype(np.float32)
+    codes = ds4.e4m3_encode(k32 / ks[..., None])
+    w = rng.uniform(0, 1, (1, H)).astype(np.float32)
+    q = ds4.round_bf16(rng.standard_normal((1, H, 576), dtype=np.float32))
+    kv = ds4.round_bf16(rng.standard_normal((1, NT, 576), dtype=np.float32))
+    t = torch.from_numpy
+    s64 = ds4.indexer_scores_fp8(qi, codes, ks, w)
+    s32 = ds4_torch.indexer_scores_fp8(t(qi[0]), t(codes[0]), t(ks[0]), t(w[0])).numpy()
+    np.testing.assert_allclose(s32, s64[0], rtol=1e-5, atol=1e-4)
+    # selection on the same float32 scores: identical sets, ties to the lower rows
+    scores = s64[0].astype(np.float32)
+    scores[700:716] = np.sort(scores)[-TOPK + 4]        # the tie block straddles the k-th place
+    want_sel = np.sort(ds4.radix_select_topk(scores, TOPK))
+    got_sel = ds4_torch.topk_rows(t(scores), TOPK).numpy()
+    np.testing.assert_array_equal(got_sel, want_sel)
+    assert (np.diff(got_sel) > 0).all()
+    tied = [r for r in got_sel if 700 <= r < 716]
+    assert tied == list(range(700, 700 + len(tied))) and 0 < len(tied) < 16
+    # the whole layer
+    sel = ds4.radix_select_topk(s32, TOPK).astype(np.int64)
+    rows = np.concatenate([np.arange(NT - WIN, NT), 4 * np.sort(sel) + 3])[None]
+    want = ds4.sparse_mla_decode(q, kv, rows, scale=576 ** -0.5)
+    got = ds4_torch.decode_layer(t(qi[0]), t(codes[0]), t(ks[0]), t(w[0]), t(q[0]), t(kv[0]), topk=TOPK, window=WIN,
+                                 scale=576 ** -0.5).numpy()
+    np.testing.assert_allclose(got, want[0], rtol=1e-5, atol=1e-5)
