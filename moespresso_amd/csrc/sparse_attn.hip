@@ -805,6 +805,7 @@ __device__ __forceinline__ f32x4_t mfma16_f16(u32x4_t a, u32x4_t b, f32x4_t c) {
 // (a count above the cases waits for everything, which is always allowed)
 #define MSPR_VM_CASE(n) case n: asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); break;
 __device__ __forceinline__ void wait_vm_dyn(int n) {
+  n = __builtin_amdgcn_readfirstlane(n);  // (the same in every lane: keeps the selection on the scalar unit)
   switch (n) {
     MSPR_VM_CASE(1) MSPR_VM_CASE(2) MSPR_VM_CASE(3) MSPR_VM_CASE(4) MSPR_VM_CASE(5) MSPR_VM_CASE(6) MSPR_VM_CASE(7)
     MSPR_VM_CASE(8) MSPR_VM_CASE(9) MSPR_VM_CASE(10) MSPR_VM_CASE(11) MSPR_VM_CASE(12) MSPR_VM_CASE(13)
