@@ -1057,7 +1057,8 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     scan_stop(cur, ids, &stop_sh[0]);
   }
   __syncthreads();
-  int n_cur = tiles_of(cur, stop_sh[0]);
+  // (read from LDS, the same in every lane: made scalar so that the tile loop's control flow is)
+  int n_cur = __builtin_amdgcn_readfirstlane(tiles_of(cur, stop_sh[0]));
   build_table(cur, 0, ids, stop_sh[0], n_cur);
   await_q();
   mask_q(cur);
