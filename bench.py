@@ -440,8 +440,11 @@ def bench_ds4_prefill(dev, gen, reps=5):
     q = torch.randn((1, H, T, 512), device=dev, generator=gen).to(torch.float16)
     raw = torch.randn((1, 1, T, 512), device=dev, generator=gen).to(torch.float16)
     comp = torch.randn((1, P, 512), device=dev, generator=gen).to(torch.float16)
-    ids = torch.stack([torch.sort(torch.randperm(P, device=dev, generator=gen)[:512]).values for _ in range(T)])
-    ids = ids[None].to(torch.int32).contiguous()
+    def distinct_sorted_ids(rows):      # 512 distinct pool rows per token, ascending
+        keys = torch.rand((T, rows), device=dev, generator=gen)
+        return keys.topk(512, dim=1).indices.sort(dim=1).values[None].to(torch.int32).contiguous()
+
+    ids = distinct_sorted_ids(P)
     sinks = torch.randn((H,), device=dev, generator=gen)
     qi = torch.randn((1, H, T, 128), device=dev, generator=gen).to(torch.float16)
     ci = torch.randn((1, P, 128), device=dev, generator=gen).to(torch.float16)
@@ -461,8 +464,7 @@ def bench_ds4_prefill(dev, gen, reps=5):
     pos_deep = 28000
     p_deep = (pos_deep + T) // 4
     comp_deep = torch.randn((1, p_deep, 512), device=dev, generator=gen).to(torch.float16)
-    ids_deep = torch.stack([torch.sort(torch.randperm(p_deep, device=dev, generator=gen)[:512]).values for _ in range(T)])
-    ids_deep = ids_deep[None].to(torch.int32).contiguous()
+    ids_deep = distinct_sorted_ids(p_deep)
     out["indexed_attention_deep_ms"] = timed(lambda: iak.indexed_mixed_attention_prefill_live_f16(
         q, raw, comp_deep, ids_deep, sinks, pos0=pos_deep, window=128, ratio=4))
     out["workload_deep"] = f"the same chunk from position {pos_deep}: {p_deep} pool rows, 640 rows per token"
