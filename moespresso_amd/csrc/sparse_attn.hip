@@ -801,23 +801,20 @@ __device__ __forceinline__ f32x4_t mfma16_f16(u32x4_t a, u32x4_t b, f32x4_t c) {
                                                 0);
 }
 
-// s_waitcnt vmcnt(n) for a wave-uniform n: at most n of this wave's vector-memory operations stay in flight
-// (a count above the cases waits for everything, which is always allowed)
-#define MSPR_VM_CASE(n) case n: asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory"); break;
+// s_waitcnt vmcnt(n') with the largest n' <= n of a few levels, for a wave-uniform n: at most n' of this wave's
+// vector-memory operations stay in flight (waiting for more than asked is always allowed). The levels are the counts
+// the prefill consumer meets: 4 or 5 (a wave's copies of one tile, every step of the steady state), 6 (with the
+// warm-up dword or the two id requests on top), 20 and above (with the sixteen output stores of the unit before).
+// A ladder of scalar compares, the common counts first: a switch over every count compiles into a chain of some
+// forty guarded blocks that a wave walks through on each wait.
 __device__ __forceinline__ void wait_vm_dyn(int n) {
   n = __builtin_amdgcn_readfirstlane(n);  // (the same in every lane: keeps the selection on the scalar unit)
-  switch (n) {
-    MSPR_VM_CASE(1) MSPR_VM_CASE(2) MSPR_VM_CASE(3) MSPR_VM_CASE(4) MSPR_VM_CASE(5) MSPR_VM_CASE(6) MSPR_VM_CASE(7)
-    MSPR_VM_CASE(8) MSPR_VM_CASE(9) MSPR_VM_CASE(10) MSPR_VM_CASE(11) MSPR_VM_CASE(12) MSPR_VM_CASE(13)
-    MSPR_VM_CASE(14) MSPR_VM_CASE(15) MSPR_VM_CASE(16) MSPR_VM_CASE(17) MSPR_VM_CASE(18) MSPR_VM_CASE(19)
-    MSPR_VM_CASE(20) MSPR_VM_CASE(21) MSPR_VM_CASE(22) MSPR_VM_CASE(23) MSPR_VM_CASE(24) MSPR_VM_CASE(25)
-    MSPR_VM_CASE(26) MSPR_VM_CASE(27) MSPR_VM_CASE(28) MSPR_VM_CASE(29) MSPR_VM_CASE(30) MSPR_VM_CASE(31)
-    MSPR_VM_CASE(32) MSPR_VM_CASE(33) MSPR_VM_CASE(34) MSPR_VM_CASE(35) MSPR_VM_CASE(36) MSPR_VM_CASE(37)
-    MSPR_VM_CASE(38) MSPR_VM_CASE(39) MSPR_VM_CASE(40)
-    default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-  }
+  if (n == 5) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+  else if (n == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+  else if (n >= 20) asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+  else if (n >= 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
-#undef MSPR_VM_CASE
 
 struct PrefillUnit {
   int b, t, hb, seq;
