@@ -972,16 +972,18 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     const int row = P / PG::kSlots, chunk = P % PG::kSlots;
     pk[j] = (P < PG::kTileSlots && chunk < 64) ? ((uint32_t)row << 16) | (uint32_t)(chunk * 16) : 0xFFFFFFFFu;
   }
-  auto copy_tile = [&](int slot, int tile, int flat) {
-    const int buf = flat & (PG::kBufs - 1);
+  // source address of each of this thread's 16-byte slots of a tile, from the row pointer table
+  auto tile_sources = [&](int slot, int tile, uint64_t (&src)[G::kPerThread]) {
     const uint64_t* rp = table + slot * PG::kTableSlots + tile * kTile;
-    uint64_t src[G::kPerThread];
 #pragma unroll
     for (int j = 0; j < G::kPerThread; j++) {
       const uint32_t p = pk[j];
       const bool act = p != 0xFFFFFFFFu;
       src[j] = rp[act ? (p >> 16) : 0] + (act ? (p & 0xFFFFu) : 0u);
     }
+  };
+  auto issue_copies = [&](const uint64_t (&src)[G::kPerThread], int flat) {
+    const int buf = flat & (PG::kBufs - 1);
     const uint32_t dst_lds = __builtin_amdgcn_readfirstlane(
         (uint32_t)(size_t)MSPR_LDS_PTR(unsigned char, kbuf + buf * G::kTileBytes + wave * 1024));
 #pragma unroll
@@ -992,6 +994,11 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
     mark_t1 = buf == 1 ? issued : mark_t1;
     mark_t2 = buf == 2 ? issued : mark_t2;
     mark_t3 = buf == 3 ? issued : mark_t3;
+  };
+  auto copy_tile = [&](int slot, int tile, int flat) {
+    uint64_t src[G::kPerThread];
+    tile_sources(slot, tile, src);
+    issue_copies(src, flat);
   };
   static_assert(PG::kBufs == 4, "ring index by mask");
   // this wave's copies of flat tile j have landed
@@ -1099,6 +1106,15 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
       if (ks & 1) so = mfma16_f16(cur_a, qf[ks], so);
       else se = mfma16_f16(cur_a, qf[ks], se);
     }
+    // The operand reads run kAhead steps in front of the matrix instructions that consume them (stated to the
+    // scheduler, which otherwise keeps only two reads in flight)
+    __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+    for (int ks = 0; ks < PG::kQSteps - kAhead; ks++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
     return se + so;
   };
 
@@ -1124,6 +1140,13 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
         oacc[mt] = mfma32<KDT>(u32x4_t{lo2.x, lo2.y, hi2.x, hi2.y}, pf[ks], oacc[mt]);
       }
     }
+    __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+    for (int i = 0; i < 6; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
   };
 
   // tile 0 is complete once every wave's copies of it are (the copies of tiles 1 and 2 stay in flight)
@@ -1154,6 +1177,20 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
         }
         if (t == 2) warm_q(nxt);
       }
+      // ---- tile s+3 (of this unit, or one of the first three of the next): its copies go out behind barrier C.
+      //      Their source addresses come out of the row pointer table in LDS; they are read here, a softmax and
+      //      a barrier ahead of their use - unless the table is the next unit's and was written only a step ago
+      //      (t < 3: no barrier has passed since), in which case they are read behind barrier C.
+      int la_slot = slot, la_tile = t + 3;
+      bool ahead = true;
+      if (la_tile >= n_cur) {
+        la_slot = slot ^ 1;
+        la_tile -= n_cur;
+        ahead = have_next;
+      }
+      const bool early = ahead && (la_slot == slot || t >= 3);
+      uint64_t la_src[G::kPerThread];
+      if (early) tile_sources(la_slot, la_tile, la_src);
       // ---- softmax weights of this wave's block: head 16 hq + c16, keys 16 kh + 4 kg + i
       float sv[4];
       {
@@ -1177,7 +1214,12 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
       // what it has issued since (the copies of tile s+2, ids, the warm-up dword, the stores of the unit before)
       if (!last || have_next) await_tile(s + 1);
       lds_barrier();  // C
-      if (__builtin_amdgcn_readfirstlane(flag[s & 1]) == s + 1) {
+      const int flagged = flag[s & 1];  // (requested here, looked at behind the copies: they do not depend on it)
+      if (ahead) {
+        if (!early) tile_sources(la_slot, la_tile, la_src);
+        issue_copies(la_src, s + 3);
+      }
+      if (__builtin_amdgcn_readfirstlane(flagged) == s + 1) {
         // ---- a key above the common maximum: the waves agree on a new one and write P^T again
         if (kg == 0) tmaxbuf[wave * 16 + c16] = tloc;
         lds_barrier();
@@ -1204,17 +1246,6 @@ __global__ __launch_bounds__(kThreads, 1) void sparse_attn_prefill_kernel(Sparse
         lds_barrier();
       }
       l_qk += (pw[0] + pw[1]) + (pw[2] + pw[3]);
-      // ---- tile s+3: of this unit, or one of the first three of the next
-      {
-        int la_slot = slot, la_tile = t + 3;
-        bool ahead = true;
-        if (la_tile >= n_cur) {
-          la_slot = slot ^ 1;
-          la_tile -= n_cur;
-          ahead = have_next;
-        }
-        if (ahead) copy_tile(la_slot, la_tile, s + 3);
-      }
       if (have_next && t == 1) {
         const int stop_pos = stop_sh[slot ^ 1];
         n_nxt = __builtin_amdgcn_readfirstlane(tiles_of(nxt, stop_pos));

@@ -32,7 +32,7 @@ def wait_level(n):
     return 6 if n >= 6 else 0
 
 
-def program(units, flagged, have_ids=True, stores_counted=None, copies_counted=None):
+def program(units, flagged, have_ids=True, stores_counted=None, copies_counted=None, early_min_t=3):
     """Events of one wave: (epoch, kind, payload...) in program order, plus the vector-memory log (tags in issue
     order) and the waits [(position in the log of the awaited operation, n passed to vmcnt, operations issued by
     then, what)]. `stores_counted` is what the wave adds to its count per unit for the output stores (the kernel:
@@ -61,11 +61,17 @@ def program(units, flagged, have_ids=True, stores_counted=None, copies_counted=N
         if counted:
             issued += copies_counted if tag[0] == "tile" else n
 
-    def copy_tile(flat):
+    def tile_sources(flat):
         act("table_read", unit_of[flat])
+
+    def issue_copies(flat):
         act("copy", flat)
         issue(("tile", flat), K_MINE, True)
         marks[("tile", flat % 4)] = (issued, len(vm) - 1)
+
+    def copy_tile(flat):
+        tile_sources(flat)
+        issue_copies(flat)
 
     def await_tile(flat):
         mark, pos = marks[("tile", flat % 4)]
@@ -123,6 +129,11 @@ def program(units, flagged, have_ids=True, stores_counted=None, copies_counted=N
                     act("stop_init", u + 1)
                 if t == 2:
                     issue(("warm", u + 1), 1, True)
+            # row pointers of tile s+3: read here unless they are the next unit's and t < 3
+            ahead = s + 3 < total and (t + 3 < n or have_next)
+            early = ahead and (t + 3 < n or t >= early_min_t)
+            if early:
+                tile_sources(s + 3)
             act("vmask_read", u)
             act("p_write", s)
             if s in flagged:
@@ -131,14 +142,16 @@ def program(units, flagged, have_ids=True, stores_counted=None, copies_counted=N
                 await_tile(s + 1)
             bar()                          # C
             act("flag_read", s)
+            if ahead:
+                if not early:
+                    tile_sources(s + 3)
+                issue_copies(s + 3)
             if s in flagged:
                 act("tmax_write", s)
                 bar()
                 act("tmax_read", s)
                 act("p_write", s)
                 bar()
-            if s + 3 < total and (t + 3 < n or have_next):
-                copy_tile(s + 3)
             if have_next and t == 1:
                 act("stop_read", u + 1)
                 act("table_build", u + 1)
@@ -254,6 +267,16 @@ def test_the_model_sees_a_wait_that_is_too_short():
     check([6, 6, 6], {0, 6, 12}, stores_counted=40)
     with pytest.raises(AssertionError, match="more in flight"):
         check([6, 6, 6], {0, 6, 12}, copies_counted=K_MINE + 1)
+
+
+def test_the_model_sees_row_pointers_read_too_early():
+    """The next unit's row pointers are written behind the barrier of step 1; reading them at the top of step 2
+    (which a unit of five tiles would do for its tile 5 = the next unit's tile 0) has no barrier in between."""
+    import pytest
+
+    check([5, 5, 5], {0, 5, 10})
+    with pytest.raises(AssertionError, match="table read before it is built"):
+        check([5, 5, 5], {0, 5, 10}, early_min_t=2)
 
 
 def test_wait_levels_never_exceed_the_count():
