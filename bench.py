@@ -35,6 +35,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0  # dense bf16 / f16
 COUNTERS_FILE = os.path.join(ROOT, "profiles", "bench_sparse_decode_layer_hbm_counters.txt")
 TRACE_FILE = os.path.join(ROOT, "profiles", "bench_all_kernels_kernel_trace_stats.txt")
 SPLIT_KERNEL_SOURCE = os.path.join(ROOT, "moespresso_amd", "csrc", "sparse_attn.hip")
@@ -419,6 +420,7 @@ def bench_q8_decode(dev, gen, reps=40):
 def bench_ds4_prefill(dev, gen, reps=5):
     """DS4 prefill-side operators at the reference's anchor chunk: 3844 tokens from position 0, 64 heads,
     961 pool rows, top-512, window 128 (wall time per call from torch events on the current stream)."""
+    from moespresso_amd import _lib
     from moespresso_amd.runtime.deepseek_v4 import attention_seam_kernel as seam
     from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
 
@@ -436,6 +438,17 @@ def bench_ds4_prefill(dev, gen, reps=5):
             torch.cuda.synchronize()
             ts.append(e0.elapsed_time(e1))
         return round(float(np.median(ts)), 4)
+
+    def kernel_ms(fn):
+        """Duration of the consumer kernel alone in the same call (events on the launch stream around the launch;
+        the per-call figure above it includes what the host needs to issue the call on an idle device)."""
+        _lib.profile_enable("sparse_split")
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        ts = _lib.profile_collect("sparse_split")
+        _lib.profile_enable()
+        return round(float(np.median(ts)), 4) if ts else None
 
     q = torch.randn((1, H, T, 512), device=dev, generator=gen).to(torch.float16)
     raw = torch.randn((1, 1, T, 512), device=dev, generator=gen).to(torch.float16)
@@ -459,6 +472,8 @@ def bench_ds4_prefill(dev, gen, reps=5):
         "workload": "3844-token chunk, 64 heads x 512, 961 pool rows, top-512, window 128 (float16 operands)",
     }
     out["partial_rope_GBps"] = round(2 * q.numel() * 2 / (out["partial_rope_query_ms"] * 1e-3) / 1e9, 1)
+    out["indexed_attention_kernel_ms"] = kernel_ms(lambda: iak.indexed_mixed_attention_prefill_live_f16(
+        q, raw, comp, ids, sinks, pos0=0, window=128, ratio=4))
     # the same chunk deep in a context: every token sees its whole window and all 512 selected rows, the pool is
     # larger than one L2 (at position 0 half of the ids lie behind the stop position and their tiles are not run)
     pos_deep = 28000
@@ -467,6 +482,11 @@ def bench_ds4_prefill(dev, gen, reps=5):
     ids_deep = distinct_sorted_ids(p_deep)
     out["indexed_attention_deep_ms"] = timed(lambda: iak.indexed_mixed_attention_prefill_live_f16(
         q, raw, comp_deep, ids_deep, sinks, pos0=pos_deep, window=128, ratio=4))
+    out["indexed_attention_deep_kernel_ms"] = kernel_ms(lambda: iak.indexed_mixed_attention_prefill_live_f16(
+        q, raw, comp_deep, ids_deep, sinks, pos0=pos_deep, window=128, ratio=4))
+    flop_deep = 4.0 * T * 640 * H * 512
+    out["indexed_attention_deep_TFLOPs"] = round(flop_deep / (out["indexed_attention_deep_kernel_ms"] * 1e-3) / 1e12, 1)
+    out["indexed_attention_deep_frac_of_2500"] = round(out["indexed_attention_deep_TFLOPs"] / MFMA_PEAK_TFLOPS, 4)
     out["workload_deep"] = f"the same chunk from position {pos_deep}: {p_deep} pool rows, 640 rows per token"
     # the other two forms of the consumer at the same chunk: float32 queries (converted to half into the workspace,
     # then the same kernel) and the banded route (band of 128 positions + every visible pool row at ratio 128)
@@ -479,6 +499,8 @@ def bench_ds4_prefill(dev, gen, reps=5):
     comp_band = torch.randn((1, p_band, 512), device=dev, generator=gen).to(torch.float16)
     ids_band = torch.arange(p_band, device=dev, dtype=torch.int32).expand(1, T, p_band).contiguous()
     out["banded_attention_deep_ms"] = timed(lambda: iak.banded_prefill_attention_live(
+        q, raw, comp_band, ids_band, sinks, pos0=pos_deep, window=128, ratio=128))
+    out["banded_attention_deep_kernel_ms"] = kernel_ms(lambda: iak.banded_prefill_attention_live(
         q, raw, comp_band, ids_band, sinks, pos0=pos_deep, window=128, ratio=128))
     out["workload_banded"] = f"banded route from position {pos_deep}: band 128, {p_band} pool rows at ratio 128, float16 queries"
     return out
