@@ -645,10 +645,13 @@ def main() -> int:
         # the same kernel in the committed kernel trace of this benchmark (graph replays, no event records around
         # the launch: events add about 1.5 us); null when the kernel source has changed since the trace was taken
         "kernel_us_traced": traced_kernel_us("sparse_attn_split_kernel<2, 576", f"{B * 16}x1x1"),
+        "frac_traced": None,
         # the whole operator (split + merge launches) against the same algorithmic bytes
         "operator_us": round(operator_us, 2),
         "operator_frac": round(MLA_BYTES_PER_SEQ * B / (operator_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
     }
+    if roofline["kernel_us_traced"]:
+        roofline["frac_traced"] = round(MLA_BYTES_PER_SEQ * B / (roofline["kernel_us_traced"] * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
     # the same kernels at the smaller batches of the configuration (first sequences of the same buffers)
     by_batch = {}
     for bsub in (1, 4):
