@@ -89,7 +89,12 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
   // tiles go out right behind, and while those fly the shares meet in LDS and every wave reads its
   // A-operand registers back from there. (Every wave fetching all of q and its 32 weights itself kept
   // the address units of a CU busy for about 3 us before the first tile could be multiplied.)
-  __shared__ __attribute__((aligned(16))) u32x4_t q_lds[2 * 8 * 64];  // [head tile][k-step][lane]: register images
+  // [head tile][k-step] register images, lane (m, g) at 33 g + m of an image of 66 entries: an image starts 32 bytes
+  // further on in the banks than the one before and its second half 16 bytes further than its first, so that the
+  // sixteen pieces of one head (eight k-steps x two halves, what sixteen consecutive threads write) fall on
+  // sixteen different 16-byte bank groups; the reads are lane-contiguous either way
+  constexpr int kImg = 66;
+  __shared__ __attribute__((aligned(16))) u32x4_t q_lds[2 * 8 * kImg];
   __shared__ float w_lds[64];
   u32x4_t qpiece[4];
 #pragma unroll
@@ -121,7 +126,7 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
     const int pc = tid + 256 * i;
     const int h = pc >> 4, c = pc & 15;
     // slot of lane (m = h % 32, g = c / 8) in the image of (head tile h / 32, k-step c % 8)
-    q_lds[((h >> 5) * 8 + (c & 7)) * 64 + 32 * (c >> 3) + (h & 31)] = h < n_heads ? qpiece[i] : u32x4_t{0u, 0u, 0u, 0u};
+    q_lds[((h >> 5) * 8 + (c & 7)) * kImg + 33 * (c >> 3) + (h & 31)] = h < n_heads ? qpiece[i] : u32x4_t{0u, 0u, 0u, 0u};
   }
   if (wave == 0) w_lds[lane] = lane < n_heads ? wmine : 0.0f;
   __syncthreads();
@@ -131,7 +136,7 @@ __global__ __launch_bounds__(256, 2) void indexer_scores_fp8_kernel(const uint16
 #pragma unroll
   for (int mt = 0; mt < 2; mt++)
 #pragma unroll
-    for (int s = 0; s < 8; s++) qa[mt][s] = q_lds[(mt * 8 + s) * 64 + lane];
+    for (int s = 0; s < 8; s++) qa[mt][s] = q_lds[(mt * 8 + s) * kImg + 33 * g + m];
   // weights of this lane's accumulator rows: head = 32mt + 8(i/4) + 4g + i%4
   float wl[2][16];
 #pragma unroll
