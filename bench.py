@@ -488,6 +488,9 @@ def bench_ds4_prefill(dev, gen, reps=5):
     out["indexed_attention_deep_TFLOPs"] = round(flop_deep / (out["indexed_attention_deep_kernel_ms"] * 1e-3) / 1e12, 1)
     out["indexed_attention_deep_frac_of_2500"] = round(out["indexed_attention_deep_TFLOPs"] / MFMA_PEAK_TFLOPS, 4)
     out["workload_deep"] = f"the same chunk from position {pos_deep}: {p_deep} pool rows, 640 rows per token"
+    ci_deep = torch.randn((1, p_deep, 128), device=dev, generator=gen).to(torch.float16)
+    out["tiled_scores_deep_ms"] = timed(lambda: iak.indexer_scores_tiled_live(qi, w, ci_deep, pos0=pos_deep, ratio=4))
+    out["tiled_scores_deep_TFLOPs"] = round(2.0 * T * p_deep * H * 128 / (out["tiled_scores_deep_ms"] * 1e-3) / 1e12, 1)
     # the other two forms of the consumer at the same chunk: float32 queries (converted to half into the workspace,
     # then the same kernel) and the banded route (band of 128 positions + every visible pool row at ratio 128)
     q32 = q.float()

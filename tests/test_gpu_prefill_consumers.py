@@ -251,7 +251,10 @@ def test_indexer_scores_tiled_live(dtype):
     from moespresso_amd.runtime.deepseek_v4 import indexed_attention_kernel as iak
 
     rng = np.random.default_rng(321)  # reference :240-247, plus a second batch entry and a larger pool
-    for (B, H, T, P, pos0) in ((1, 8, 5, 19, 0), (2, 64, 37, 300, 250), (1, 48, 9, 33, 1000)):
+    # (the last two: several tiles per workgroup with the visible prefix ending inside a block; five tiles per
+    # workgroup, all visible, a ragged last block)
+    for (B, H, T, P, pos0) in ((1, 8, 5, 19, 0), (2, 64, 37, 300, 250), (1, 48, 9, 33, 1000), (1, 64, 130, 1000, 1500),
+                               (1, 64, 300, 1500, 9000)):
         q = rng.standard_normal((B, H, T, 128), dtype=np.float32)
         w = (rng.standard_normal((B, T, H), dtype=np.float32) * (H ** -0.5) * (128 ** -0.5)).astype(np.float32)
         comp = rng.standard_normal((B, P, 128), dtype=np.float32)
