@@ -472,6 +472,9 @@ def bench_ds4_prefill(dev, gen, reps=5):
         "workload": "3844-token chunk, 64 heads x 512, 961 pool rows, top-512, window 128 (float16 operands)",
     }
     out["partial_rope_GBps"] = round(2 * q.numel() * 2 / (out["partial_rope_query_ms"] * 1e-3) / 1e9, 1)
+    from moespresso_amd.runtime.deepseek_v4 import indexer_score_kernel as isk
+    sc = torch.randn((T, P), device=dev, generator=gen)
+    out["topk_512_ms"] = timed(lambda: isk.topk_select(sc, 512))
     out["indexed_attention_kernel_ms"] = kernel_ms(lambda: iak.indexed_mixed_attention_prefill_live_f16(
         q, raw, comp, ids, sinks, pos0=0, window=128, ratio=4))
     # the same chunk deep in a context: every token sees its whole window and all 512 selected rows, the pool is
@@ -490,6 +493,8 @@ def bench_ds4_prefill(dev, gen, reps=5):
     out["workload_deep"] = f"the same chunk from position {pos_deep}: {p_deep} pool rows, 640 rows per token"
     ci_deep = torch.randn((1, p_deep, 128), device=dev, generator=gen).to(torch.float16)
     out["tiled_scores_deep_ms"] = timed(lambda: iak.indexer_scores_tiled_live(qi, w, ci_deep, pos0=pos_deep, ratio=4))
+    sc_deep = torch.randn((T, p_deep), device=dev, generator=gen)
+    out["topk_512_deep_ms"] = timed(lambda: isk.topk_select(sc_deep, 512))
     out["tiled_scores_deep_TFLOPs"] = round(2.0 * T * p_deep * H * 128 / (out["tiled_scores_deep_ms"] * 1e-3) / 1e12, 1)
     # the other two forms of the consumer at the same chunk: float32 queries (converted to half into the workspace,
     # then the same kernel) and the banded route (band of 128 positions + every visible pool row at ratio 128)

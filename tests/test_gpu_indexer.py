@@ -312,7 +312,11 @@ def test_fused_decode_prep_integer_inputs_are_bitexact_end_to_end():
 
 
 @pytest.mark.parametrize("shape_k", [((5,), 1), ((5,), 5), ((600,), 512), ((3, 977), 512), ((2, 8192), 2048),
-                                     ((16, 32768), 2048), ((2, 70001), 2048), ((1, 32768), 32768)])
+                                     ((16, 32768), 2048), ((2, 70001), 2048), ((1, 32768), 32768),
+                                     # rows of up to 2048 scores take a kernel of their own (one 256-thread workgroup
+                                     # a row): its two widths, their boundaries, many rows, k = all rows
+                                     ((70, 961), 512), ((9, 1024), 1024), ((5, 1025), 7), ((4, 2048), 2048),
+                                     ((3, 2049), 100), ((300, 64), 33), ((130, 4096), 512), ((129, 7961), 512), ((128, 8192), 8000)])
 def test_topk_select_bitexact(shape_k):
     shape, k = shape_k
     rng = np.random.default_rng(sum(shape) + k)
