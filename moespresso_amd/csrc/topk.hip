@@ -385,7 +385,10 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
                                                                  int64_t score_stride, int n_rows, int topk,
                                                                  int sample_rank, int32_t* __restrict__ sel_all) {
   // The staging area for the load (C*1024 keys) is reused for the histogram copies afterwards.
-  constexpr int kStageWords = C * kThreads > 256 * kCopies ? C * kThreads : 256 * kCopies;
+  // copies of the full-pass histograms: one per lane where the staging area is that large anyway; 32 (lanes l and
+  // l + 32 share one) for the short-row instance, whose LDS then lets two workgroups share a CU
+  constexpr int kCp = C * kThreads >= 256 * kCopies ? kCopies : kCopies / 2;
+  constexpr int kStageWords = C * kThreads > 256 * kCp ? C * kThreads : 256 * kCp;
   __shared__ __attribute__((aligned(16))) uint32_t stage[kStageWords];
   uint32_t* hist = stage;                   // [bin][copy]
   __shared__ uint32_t totals[256];
@@ -569,7 +572,7 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
 
   {
     u32x4_t* h4 = reinterpret_cast<u32x4_t*>(hist);
-    for (int i = tid; i < 256 * kCopies / 4; i += kThreads) h4[i] = u32x4_t{0u, 0u, 0u, 0u};
+    for (int i = tid; i < 256 * kCp / 4; i += kThreads) h4[i] = u32x4_t{0u, 0u, 0u, 0u};
     if (tid < 512) (&small_hist[0][0])[tid] = 0u;
     if (tid == 0) list_n = 0u;
   }
@@ -584,17 +587,18 @@ __global__ __launch_bounds__(kThreads) void topk_blocked_kernel(const float* __r
 #pragma unroll
     for (int i = 0; i < C; i++) {
       const uint32_t key = kreg[i];
-      if (pass == 0 || (key & mask_hi) == prefix) atomicAdd(&hist[((key >> shift) & 0xFFu) * kCopies + lane], 1u);
+      if (pass == 0 || (key & mask_hi) == prefix)
+        atomicAdd(&hist[((key >> shift) & 0xFFu) * kCp + (lane & (kCp - 1))], 1u);
     }
     __syncthreads();
-    // totals[bin] = sum over copies: four threads per bin, 16 copies each as four 16-byte reads
+    // totals[bin] = sum over copies: four threads per bin, a quarter of the copies each as 16-byte reads
     // (rotated so that 16 neighbouring lanes cover all 16 bank groups), zeroed behind the read
     {
       const int bin = tid >> 2, q = tid & 3;
       uint32_t sum = 0u;
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        u32x4_t* p = reinterpret_cast<u32x4_t*>(&hist[bin * kCopies + q * 16 + 4 * ((j + (tid >> 2)) & 3)]);
+      for (int j = 0; j < kCp / 16; j++) {
+        u32x4_t* p = reinterpret_cast<u32x4_t*>(&hist[bin * kCp + q * (kCp / 4) + 4 * ((j + (tid >> 2)) & (kCp / 16 - 1))]);
         const u32x4_t v = *p;
         *p = u32x4_t{0u, 0u, 0u, 0u};
         sum += v.x + v.y + v.z + v.w;
